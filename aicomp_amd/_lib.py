@@ -1,0 +1,78 @@
+"""ctypes binding of libaicomp_kv.so (the C ABI declared in include/aicomp_kv.h).
+
+There is no CPU fallback: if the HIP library is missing, loading raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import threading
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libaicomp_kv.so")
+
+# every symbol include/aicomp_kv.h declares
+SYMBOLS = (
+    "aicomp_kv_version",
+    "aicomp_kv_last_error",
+    "aicomp_kv_append",
+    "aicomp_paged_decode_attn",
+    "aicomp_paged_decode_workspace_bytes",
+    "aicomp_paged_decode_partition_size",
+    "aicomp_paged_prefill_attn",
+)
+
+F32, BF16, FP8_E4M3 = 0, 1, 2
+
+_lock = threading.Lock()
+_lib = None
+
+
+class LibraryMissing(RuntimeError):
+    pass
+
+
+def _declare(lib: C.CDLL) -> None:
+    vp, i64, i32, f32, sz = C.c_void_p, C.c_int64, C.c_int, C.c_float, C.c_size_t
+    lib.aicomp_kv_version.restype = i32
+    lib.aicomp_kv_version.argtypes = []
+    lib.aicomp_kv_last_error.restype = C.c_char_p
+    lib.aicomp_kv_last_error.argtypes = []
+    lib.aicomp_kv_append.restype = i32
+    lib.aicomp_kv_append.argtypes = [vp, vp, i64, i64, vp, vp, vp, i64, i32, i32, i32, i64,
+                                     i32, i32, vp, vp, vp]
+    lib.aicomp_paged_decode_attn.restype = i32
+    lib.aicomp_paged_decode_attn.argtypes = [vp, vp, vp, vp, vp, i64, vp, i32, i32, i32, i32,
+                                             i32, i32, i64, f32, i32, i32, vp, vp, i32, vp, sz, vp]
+    lib.aicomp_paged_decode_workspace_bytes.restype = sz
+    lib.aicomp_paged_decode_workspace_bytes.argtypes = [i32] * 9
+    lib.aicomp_paged_decode_partition_size.restype = i32
+    lib.aicomp_paged_decode_partition_size.argtypes = [i32] * 8
+    lib.aicomp_paged_prefill_attn.restype = i32
+    lib.aicomp_paged_prefill_attn.argtypes = [vp, vp, vp, vp, vp, i64, vp, vp, i32, i64, i32,
+                                              i32, i32, i32, i32, i32, i64, f32, i32, i32,
+                                              vp, vp, vp]
+
+
+def load() -> C.CDLL:
+    """Load the HIP library built by ``python -m aicomp_amd.build``."""
+    global _lib
+    with _lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise LibraryMissing(
+                    f"{LIB_PATH} is missing: build it with `python -m aicomp_amd.build` "
+                    "(hipcc, gfx950). There is no CPU fallback for this path.")
+            lib = C.CDLL(LIB_PATH)
+            for s in SYMBOLS:
+                if not hasattr(lib, s):
+                    raise LibraryMissing(f"{LIB_PATH} does not export {s}")
+            _declare(lib)
+            _lib = lib
+        return _lib
+
+
+def check(rc: int, lib: C.CDLL) -> None:
+    if rc != 0:
+        msg = lib.aicomp_kv_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"aicomp_kv error {rc}: {msg}")

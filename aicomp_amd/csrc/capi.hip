@@ -1,0 +1,203 @@
+// extern "C" entry points: argument validation and kernel dispatch.
+// The declarations, with the reference interfaces they replace, are in
+// include/aicomp_kv.h.
+#include "common.h"
+
+#include <string.h>
+
+namespace aicomp {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int launch_kv_append(const void* key, const void* value, int64_t token_stride, int64_t head_stride,
+                     void* k_pool, void* v_pool, const int64_t* slot_mapping, int64_t T, int hkv,
+                     int d, int bs, int64_t num_blocks, int in_dtype, int pool_dtype,
+                     const float* k_scale, const float* v_scale, hipStream_t stream);
+
+struct PrefillArgs;
+bool prefill_mfma_supported(const DecodeArgs& a, int max_q_len);
+int launch_prefill_mfma(const DecodeArgs& a, int max_q_len);
+
+static int check_common(int hq, int hkv, int d, int bs, int max_blocks, int64_t num_blocks,
+                        int q_dtype, int kv_dtype, const float* k_scale, const float* v_scale,
+                        const char* who) {
+    AICOMP_REQUIRE(hq > 0 && hkv > 0 && hq % hkv == 0, AICOMP_KV_EINVAL,
+                   "%s: %d query heads are not a multiple of %d KV heads", who, hq, hkv);
+    AICOMP_REQUIRE(d > 0 && bs > 0 && max_blocks >= 0 && num_blocks > 0, AICOMP_KV_EINVAL,
+                   "%s: bad sizes (head_dim %d, block_size %d, max_blocks %d, num_blocks %lld)",
+                   who, d, bs, max_blocks, (long long)num_blocks);
+    AICOMP_REQUIRE(dtype_size(q_dtype) && dtype_size(kv_dtype), AICOMP_KV_EINVAL,
+                   "%s: unknown element type (query %d, pool %d)", who, q_dtype, kv_dtype);
+    if (kv_dtype == AICOMP_KV_FP8_E4M3)
+        AICOMP_REQUIRE(k_scale && v_scale, AICOMP_KV_EINVAL,
+                       "%s: an fp8 pool needs k_scale and v_scale", who);
+    return AICOMP_KV_OK;
+}
+
+static int auto_partition(int64_t rows, int hkv, int bs, int max_blocks) {
+    const int64_t max_ctx = (int64_t)max_blocks * bs;
+    int ps = 512;
+    // few work items: smaller partitions fill the 256 CUs sooner
+    if (rows * hkv * ((max_ctx + 511) / 512) < 1024) ps = 256;
+    ps = (ps + bs - 1) / bs * bs;
+    return ps;
+}
+
+}  // namespace aicomp
+
+using namespace aicomp;
+
+extern "C" {
+
+int aicomp_kv_version(void) { return 100; }
+
+const char* aicomp_kv_last_error(void) { return g_err; }
+
+int aicomp_kv_append(const void* key, const void* value, int64_t kv_token_stride,
+                     int64_t kv_head_stride, void* k_pool, void* v_pool,
+                     const int64_t* slot_mapping, int64_t num_tokens, int num_kv_heads,
+                     int head_dim, int block_size, int64_t num_blocks, int in_dtype,
+                     int pool_dtype, const float* k_scale, const float* v_scale, void* stream) {
+    AICOMP_REQUIRE(num_tokens >= 0, AICOMP_KV_EINVAL, "kv_append: negative token count");
+    if (num_tokens == 0) return AICOMP_KV_OK;
+    AICOMP_REQUIRE(key && value && k_pool && v_pool && slot_mapping, AICOMP_KV_EINVAL,
+                   "kv_append: null pointer");
+    AICOMP_REQUIRE(num_kv_heads > 0 && head_dim > 0 && block_size > 0 && num_blocks > 0,
+                   AICOMP_KV_EINVAL, "kv_append: bad sizes (Hkv %d, D %d, BS %d, blocks %lld)",
+                   num_kv_heads, head_dim, block_size, (long long)num_blocks);
+    AICOMP_REQUIRE(dtype_size(in_dtype) && dtype_size(pool_dtype), AICOMP_KV_EINVAL,
+                   "kv_append: unknown element type (in %d, pool %d)", in_dtype, pool_dtype);
+    AICOMP_REQUIRE(kv_head_stride >= head_dim && kv_token_stride >= 0, AICOMP_KV_EINVAL,
+                   "kv_append: strides (%lld, %lld) overlap rows of %d elements",
+                   (long long)kv_token_stride, (long long)kv_head_stride, head_dim);
+    return launch_kv_append(key, value, kv_token_stride, kv_head_stride, k_pool, v_pool,
+                            slot_mapping, num_tokens, num_kv_heads, head_dim, block_size,
+                            num_blocks, in_dtype, pool_dtype, k_scale, v_scale,
+                            (hipStream_t)stream);
+}
+
+int aicomp_paged_decode_partition_size(int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                                       int block_size, int max_blocks_per_seq, int q_dtype,
+                                       int kv_dtype) {
+    (void)num_q_heads; (void)head_dim; (void)q_dtype; (void)kv_dtype;
+    if (batch <= 0 || num_kv_heads <= 0 || block_size <= 0 || max_blocks_per_seq <= 0) return 0;
+    return auto_partition(batch, num_kv_heads, block_size, max_blocks_per_seq);
+}
+
+static int resolve_parts(int64_t rows, int hkv, int bs, int max_blocks, int& partition_size) {
+    if (partition_size <= 0) partition_size = auto_partition(rows, hkv, bs, max_blocks);
+    const int64_t max_ctx = (int64_t)max_blocks * bs;
+    int64_t parts = (max_ctx + partition_size - 1) / partition_size;
+    return (int)(parts < 1 ? 1 : parts);
+}
+
+size_t aicomp_paged_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads,
+                                           int head_dim, int block_size, int max_blocks_per_seq,
+                                           int q_dtype, int kv_dtype, int partition_size) {
+    (void)q_dtype; (void)kv_dtype;
+    if (batch <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || block_size <= 0 ||
+        max_blocks_per_seq <= 0)
+        return 0;
+    const int parts = resolve_parts(batch, num_kv_heads, block_size, max_blocks_per_seq, partition_size);
+    if (parts <= 1) return 0;
+    return split_workspace_bytes(batch, num_q_heads, head_dim, parts);
+}
+
+int aicomp_paged_decode_attn(void* out, const void* query, const void* k_pool, const void* v_pool,
+                             const int32_t* block_table, int64_t block_table_stride,
+                             const int32_t* context_lens, int batch, int num_q_heads,
+                             int num_kv_heads, int head_dim, int block_size,
+                             int max_blocks_per_seq, int64_t num_blocks, float scale, int q_dtype,
+                             int kv_dtype, const float* k_scale, const float* v_scale,
+                             int partition_size, void* workspace, size_t workspace_bytes,
+                             void* stream) {
+    AICOMP_REQUIRE(batch >= 0, AICOMP_KV_EINVAL, "paged_decode_attn: negative batch");
+    if (batch == 0) return AICOMP_KV_OK;
+    AICOMP_REQUIRE(out && query && k_pool && v_pool && block_table && context_lens,
+                   AICOMP_KV_EINVAL, "paged_decode_attn: null pointer");
+    int rc = check_common(num_q_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq,
+                          num_blocks, q_dtype, kv_dtype, k_scale, v_scale, "paged_decode_attn");
+    if (rc) return rc;
+    AICOMP_REQUIRE(max_blocks_per_seq > 0 && block_table_stride >= max_blocks_per_seq,
+                   AICOMP_KV_EINVAL, "paged_decode_attn: block table stride %lld < width %d",
+                   (long long)block_table_stride, max_blocks_per_seq);
+    AICOMP_REQUIRE(partition_size >= 0 && partition_size % block_size == 0, AICOMP_KV_EINVAL,
+                   "paged_decode_attn: partition_size %d is not a multiple of block_size %d",
+                   partition_size, block_size);
+    DecodeArgs a;
+    memset(&a, 0, sizeof(a));
+    a.out = out; a.query = query; a.k_pool = k_pool; a.v_pool = v_pool;
+    a.block_table = block_table; a.block_table_stride = block_table_stride;
+    a.context_lens = context_lens; a.cu_q_lens = nullptr;
+    a.num_seqs = batch; a.rows = batch;
+    a.hq = num_q_heads; a.hkv = num_kv_heads; a.d = head_dim; a.bs = block_size;
+    a.max_blocks = max_blocks_per_seq; a.num_blocks = num_blocks;
+    a.scale = scale; a.q_dtype = q_dtype; a.kv_dtype = kv_dtype;
+    a.k_scale = kv_dtype == AICOMP_KV_FP8_E4M3 ? k_scale : nullptr;
+    a.v_scale = kv_dtype == AICOMP_KV_FP8_E4M3 ? v_scale : nullptr;
+    a.partition_size = partition_size;
+    a.num_parts = resolve_parts(batch, num_kv_heads, block_size, max_blocks_per_seq, a.partition_size);
+    a.stream = (hipStream_t)stream;
+    if (a.num_parts > 1) {
+        const size_t need = split_workspace_bytes(a.rows, a.hq, a.d, a.num_parts);
+        AICOMP_REQUIRE(workspace && workspace_bytes >= need, AICOMP_KV_EWORKSPACE,
+                       "paged_decode_attn: workspace of %zu bytes needed, %zu given", need,
+                       workspace ? workspace_bytes : (size_t)0);
+        AICOMP_REQUIRE((uintptr_t)workspace % 16 == 0, AICOMP_KV_EINVAL,
+                       "paged_decode_attn: workspace must be 16-byte aligned");
+        a.ws = split_workspace_view(workspace, a.rows, a.hq, a.d, a.num_parts);
+    }
+    if (decode_mfma_supported(a)) return launch_decode_mfma(a);
+    return launch_decode_generic(a);
+}
+
+int aicomp_paged_prefill_attn(void* out, const void* query, const void* k_pool, const void* v_pool,
+                              const int32_t* block_table, int64_t block_table_stride,
+                              const int32_t* context_lens, const int32_t* cu_q_lens, int num_seqs,
+                              int64_t total_q, int max_q_len, int num_q_heads, int num_kv_heads,
+                              int head_dim, int block_size, int max_blocks_per_seq,
+                              int64_t num_blocks, float scale, int q_dtype, int kv_dtype,
+                              const float* k_scale, const float* v_scale, void* stream) {
+    AICOMP_REQUIRE(num_seqs >= 0 && total_q >= 0, AICOMP_KV_EINVAL,
+                   "paged_prefill_attn: negative sizes");
+    if (num_seqs == 0 || total_q == 0) return AICOMP_KV_OK;
+    AICOMP_REQUIRE(out && query && k_pool && v_pool && block_table && context_lens && cu_q_lens,
+                   AICOMP_KV_EINVAL, "paged_prefill_attn: null pointer");
+    int rc = check_common(num_q_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq,
+                          num_blocks, q_dtype, kv_dtype, k_scale, v_scale, "paged_prefill_attn");
+    if (rc) return rc;
+    AICOMP_REQUIRE(max_q_len > 0 && max_q_len <= total_q, AICOMP_KV_EINVAL,
+                   "paged_prefill_attn: max_q_len %d out of range (total %lld)", max_q_len,
+                   (long long)total_q);
+    AICOMP_REQUIRE(max_blocks_per_seq > 0 && block_table_stride >= max_blocks_per_seq,
+                   AICOMP_KV_EINVAL, "paged_prefill_attn: block table stride %lld < width %d",
+                   (long long)block_table_stride, max_blocks_per_seq);
+    DecodeArgs a;
+    memset(&a, 0, sizeof(a));
+    a.out = out; a.query = query; a.k_pool = k_pool; a.v_pool = v_pool;
+    a.block_table = block_table; a.block_table_stride = block_table_stride;
+    a.context_lens = context_lens; a.cu_q_lens = cu_q_lens;
+    a.num_seqs = num_seqs; a.rows = total_q;
+    a.hq = num_q_heads; a.hkv = num_kv_heads; a.d = head_dim; a.bs = block_size;
+    a.max_blocks = max_blocks_per_seq; a.num_blocks = num_blocks;
+    a.scale = scale; a.q_dtype = q_dtype; a.kv_dtype = kv_dtype;
+    a.k_scale = kv_dtype == AICOMP_KV_FP8_E4M3 ? k_scale : nullptr;
+    a.v_scale = kv_dtype == AICOMP_KV_FP8_E4M3 ? v_scale : nullptr;
+    a.stream = (hipStream_t)stream;
+    if (prefill_mfma_supported(a, max_q_len)) return launch_prefill_mfma(a, max_q_len);
+    // shapes outside the MFMA kernel: every query row as its own unsplit
+    // attention problem over its causal prefix (vector-ALU kernel)
+    a.partition_size = (int)(((int64_t)max_blocks_per_seq * block_size + block_size - 1) /
+                             block_size * block_size);
+    a.num_parts = 1;
+    return launch_decode_generic(a);
+}
+
+}  // extern "C"

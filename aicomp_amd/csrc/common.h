@@ -1,0 +1,156 @@
+// Shared device/host helpers for the paged KV-cache attention kernels (gfx950).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/aicomp_kv.h"
+
+namespace aicomp {
+
+// ---------------------------------------------------------------- errors ---
+void set_error(const char* fmt, ...);
+
+#define AICOMP_REQUIRE(cond, code, ...)                 \
+    do {                                                \
+        if (!(cond)) {                                  \
+            ::aicomp::set_error(__VA_ARGS__);           \
+            return (code);                              \
+        }                                               \
+    } while (0)
+
+#define AICOMP_HIP_LAUNCH_CHECK()                                              \
+    do {                                                                       \
+        hipError_t e__ = hipGetLastError();                                    \
+        if (e__ != hipSuccess) {                                               \
+            ::aicomp::set_error("HIP launch failed: %s", hipGetErrorString(e__)); \
+            return AICOMP_KV_EHIP;                                             \
+        }                                                                      \
+    } while (0)
+
+inline int dtype_size(int dt) {
+    switch (dt) {
+        case AICOMP_KV_F32: return 4;
+        case AICOMP_KV_BF16: return 2;
+        case AICOMP_KV_FP8_E4M3: return 1;
+        default: return 0;
+    }
+}
+
+// --------------------------------------------------------- element types ---
+struct bf16_t { uint16_t bits; };
+struct fp8_t { uint8_t bits; };
+
+constexpr int WAVE = 64;
+constexpr float LOG2E = 1.4426950408889634f;
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) {
+    return __uint_as_float(((uint32_t)b) << 16);
+}
+
+// round-to-nearest-even, NaN kept quiet (same rule as torch's bfloat16 cast)
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+// OCP e4m3 code -> float: gfx950's hardware conversion (byte 0 of the word)
+__device__ __forceinline__ float fp8_to_f32(uint8_t c) {
+    return __builtin_amdgcn_cvt_f32_fp8((int)c, 0);
+}
+
+// 16 raw bytes -> floats, by storage type
+template <typename T> struct Vec16;
+
+template <> struct Vec16<float> {
+    static constexpr int N = 4;
+    __device__ __forceinline__ static void unpack(const uint4& r, float* f) {
+        f[0] = __uint_as_float(r.x); f[1] = __uint_as_float(r.y);
+        f[2] = __uint_as_float(r.z); f[3] = __uint_as_float(r.w);
+    }
+};
+template <> struct Vec16<bf16_t> {
+    static constexpr int N = 8;
+    __device__ __forceinline__ static void unpack(const uint4& r, float* f) {
+        const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = __uint_as_float(w[i] << 16);
+            f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+};
+template <> struct Vec16<fp8_t> {
+    static constexpr int N = 16;
+    __device__ __forceinline__ static void unpack(const uint4& r, float* f) {
+        const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            auto lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], false);
+            auto hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], true);
+            f[4 * i] = lo[0]; f[4 * i + 1] = lo[1];
+            f[4 * i + 2] = hi[0]; f[4 * i + 3] = hi[1];
+        }
+    }
+};
+
+template <typename T> __device__ __forceinline__ float load_elem(const T* p);
+template <> __device__ __forceinline__ float load_elem<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float load_elem<bf16_t>(const bf16_t* p) { return bf16_to_f32(p->bits); }
+
+template <typename T> __device__ __forceinline__ void store_elem(T* p, float v);
+template <> __device__ __forceinline__ void store_elem<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void store_elem<bf16_t>(bf16_t* p, float v) { p->bits = f32_to_bf16(v); }
+
+// ------------------------------------------------- split-K workspace view ---
+// part_acc [rows][Hq][P][D] float : sum_j 2^(s_j - m) v_j   (not normalised)
+// part_ml  [rows][Hq][P][2] float : m (log2 domain), l = sum_j 2^(s_j - m)
+struct SplitWorkspace {
+    float* acc;
+    float* ml;
+};
+
+inline size_t split_workspace_bytes(int64_t rows, int hq, int d, int parts) {
+    return (size_t)rows * hq * parts * (size_t)(d + 2) * sizeof(float);
+}
+inline SplitWorkspace split_workspace_view(void* ws, int64_t rows, int hq, int d, int parts) {
+    SplitWorkspace v;
+    v.acc = (float*)ws;
+    v.ml = v.acc + (size_t)rows * hq * parts * d;
+    return v;
+}
+
+// ------------------------------------------------------- kernel launchers ---
+struct DecodeArgs {
+    void* out;
+    const void* query;
+    const void* k_pool;
+    const void* v_pool;
+    const int32_t* block_table;
+    int64_t block_table_stride;
+    const int32_t* context_lens;
+    const int32_t* cu_q_lens;   // NULL: one query row per sequence (decode)
+    int num_seqs;
+    int64_t rows;               // query rows (== num_seqs for decode)
+    int hq, hkv, d, bs, max_blocks;
+    int64_t num_blocks;
+    float scale;
+    int q_dtype, kv_dtype;
+    const float* k_scale;
+    const float* v_scale;
+    int partition_size;         // tokens, multiple of bs
+    int num_parts;              // ceil(max_blocks*bs / partition_size)
+    SplitWorkspace ws;
+    hipStream_t stream;
+};
+
+int launch_decode_generic(const DecodeArgs& a);
+bool decode_mfma_supported(const DecodeArgs& a);
+int launch_decode_mfma(const DecodeArgs& a);
+int launch_split_reduce(const DecodeArgs& a);
+
+}  // namespace aicomp

@@ -1,0 +1,347 @@
+// Generic paged attention kernel (vector ALU): any supported storage type,
+// head_dim 64/128/256, any GQA group, any block size.  It is the path for
+// shapes the MFMA kernels do not cover (fp32 pools, head_dim != 128, block
+// sizes other than 16) and the split-K reduce shared by every decode kernel.
+//
+// Replaces  F.scaled_dot_product_attention(query, full_key, full_value,
+//           attn_mask=None, is_causal=False)       opt_prime/opt_prime/kv_cache.py:397-403
+// (and, with cu_q_lens, the is_causal=True prefill of kv_cache.py:404-415, one
+// query row at a time) reading K/V through the block table instead of from the
+// .contiguous() prefix copy of kv_cache.py:391-392.
+//
+// Work split: one workgroup (4 waves) per (query row, KV head, partition).
+// A K/V row of D elements is read by LPR consecutive lanes with one 16-byte
+// (8-byte for fp8) load each, so a wave reads 64/LPR whole rows per load:
+// full-line, coalesced requests.  Every lane group keeps its own online-softmax
+// state (running max, sum, accumulator) for the tokens it visits; the groups
+// are merged with wave shuffles, the waves through LDS.  All G query heads of
+// the KV head share each loaded K/V chunk.
+#include "common.h"
+
+namespace aicomp {
+
+template <typename KV_T> struct KvLoad;
+template <> struct KvLoad<float> {
+    static constexpr int N = 4;
+    __device__ __forceinline__ static void load(const float* p, float* f) {
+        uint4 r = *reinterpret_cast<const uint4*>(p);
+        Vec16<float>::unpack(r, f);
+    }
+};
+template <> struct KvLoad<bf16_t> {
+    static constexpr int N = 8;
+    __device__ __forceinline__ static void load(const bf16_t* p, float* f) {
+        uint4 r = *reinterpret_cast<const uint4*>(p);
+        Vec16<bf16_t>::unpack(r, f);
+    }
+};
+template <> struct KvLoad<fp8_t> {
+    static constexpr int N = 8;
+    __device__ __forceinline__ static void load(const fp8_t* p, float* f) {
+        uint2 r = *reinterpret_cast<const uint2*>(p);
+        const uint32_t w[2] = {r.x, r.y};
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            auto lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], false);
+            auto hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], true);
+            f[4 * i] = lo[0]; f[4 * i + 1] = lo[1];
+            f[4 * i + 2] = hi[0]; f[4 * i + 3] = hi[1];
+        }
+    }
+};
+
+struct GenericParams {
+    void* out;
+    const void* query;
+    const void* k_pool;
+    const void* v_pool;
+    const int32_t* block_table;
+    int64_t block_table_stride;
+    const int32_t* context_lens;
+    const int32_t* cu_q_lens;
+    int num_seqs;
+    int hq, hkv, group, bs;
+    int64_t num_blocks;
+    float qk_mul;               // scale * log2(e)
+    const float* k_scale;
+    const float* v_scale;
+    int partition_size, num_parts;
+    float* ws_acc;
+    float* ws_ml;
+};
+
+// sequence and attended length of a query row
+__device__ __forceinline__ void row_info(int64_t row, const int32_t* cu, const int32_t* ctx,
+                                         int num_seqs, int& seq, int& len) {
+    if (cu == nullptr) {
+        seq = (int)row;
+        len = ctx[row];
+    } else {
+        int lo = 0, hi = num_seqs;       // largest s with cu[s] <= row
+        while (hi - lo > 1) {
+            int mid = (lo + hi) >> 1;
+            if (cu[mid] <= row) lo = mid; else hi = mid;
+        }
+        seq = lo;
+        int n = cu[lo + 1] - cu[lo];
+        int i = (int)(row - cu[lo]);
+        len = ctx[lo] - n + i + 1;       // bottom-right aligned causal mask
+    }
+    if (len < 0) len = 0;
+}
+
+constexpr float NEG_BIG = -1.0e30f;
+
+template <typename KV_T, typename Q_T, int D, int GMAX>
+__global__ void __launch_bounds__(256)
+paged_attn_generic_kernel(GenericParams p) {
+    constexpr int N = KvLoad<KV_T>::N;
+    constexpr int LPR = D / N;            // lanes per K/V row
+    constexpr int TPW = WAVE / LPR;       // rows per wave per load
+    constexpr int NW = 4;
+    static_assert(LPR >= 1 && LPR <= 64 && (LPR & (LPR - 1)) == 0, "row must split over 2^k lanes");
+
+    const int64_t row = blockIdx.x;
+    const int groups_per_kv = (p.group + GMAX - 1) / GMAX;
+    const int kvh = blockIdx.y / groups_per_kv;
+    const int g0 = (blockIdx.y % groups_per_kv) * GMAX;      // first head of the group handled here
+    const int gn = min(GMAX, p.group - g0);
+    const int part = blockIdx.z;
+
+    int seq, len;
+    row_info(row, p.cu_q_lens, p.context_lens, p.num_seqs, seq, len);
+    const int start = part * p.partition_size;
+    const int end = min(len, start + p.partition_size);
+    const int tid = threadIdx.x;
+    const int head0 = kvh * p.group + g0;
+
+    if (start >= end) {
+        // nothing here; an unsplit call still owes the caller a defined output
+        if (p.num_parts == 1) {
+            Q_T* o = (Q_T*)p.out + (row * p.hq + head0) * D;
+            for (int i = tid; i < gn * D; i += blockDim.x) store_elem<Q_T>(o + i, 0.f);
+        }
+        return;
+    }
+
+    const int w = tid / WAVE, lane = tid % WAVE;
+    const int sub = lane / LPR, lr = lane % LPR;
+
+    float q[GMAX][N];
+    {
+        const float mul = p.qk_mul * (p.k_scale ? p.k_scale[kvh] : 1.f);
+        const Q_T* qp = (const Q_T*)p.query + (row * p.hq + head0) * D + lr * N;
+#pragma unroll
+        for (int g = 0; g < GMAX; ++g)
+#pragma unroll
+            for (int e = 0; e < N; ++e)
+                q[g][e] = (g < gn) ? load_elem<Q_T>(qp + g * D + e) * mul : 0.f;
+    }
+
+    float m[GMAX], l[GMAX], acc[GMAX][N];
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) {
+        m[g] = NEG_BIG; l[g] = 0.f;
+#pragma unroll
+        for (int e = 0; e < N; ++e) acc[g][e] = 0.f;
+    }
+
+    const int32_t* table = p.block_table + (int64_t)seq * p.block_table_stride;
+    const KV_T* kp = (const KV_T*)p.k_pool;
+    const KV_T* vp = (const KV_T*)p.v_pool;
+    const int steps = (end - start + NW * TPW - 1) / (NW * TPW);
+
+    for (int it = 0; it < steps; ++it) {
+        const int tok = start + it * NW * TPW + w * TPW + sub;
+        const bool valid = tok < end;
+        float kf[N], vf[N];
+        int64_t base = 0;
+        if (valid) {
+            int64_t blk = table[tok / p.bs];
+            blk = blk < 0 ? 0 : (blk >= p.num_blocks ? p.num_blocks - 1 : blk);  // never leave the pool
+            base = ((blk * p.hkv + kvh) * p.bs + tok % p.bs) * D + lr * N;
+            KvLoad<KV_T>::load(kp + base, kf);
+            KvLoad<KV_T>::load(vp + base, vf);
+        } else {
+#pragma unroll
+            for (int e = 0; e < N; ++e) { kf[e] = 0.f; vf[e] = 0.f; }
+        }
+#pragma unroll
+        for (int g = 0; g < GMAX; ++g) {
+            float s = 0.f;
+#pragma unroll
+            for (int e = 0; e < N; ++e) s = fmaf(q[g][e], kf[e], s);
+#pragma unroll
+            for (int o = 1; o < LPR; o <<= 1) s += __shfl_xor(s, o);
+            const float m_new = valid ? fmaxf(m[g], s) : m[g];
+            const float alpha = exp2f(m[g] - m_new);
+            const float pr = valid ? exp2f(s - m_new) : 0.f;
+            m[g] = m_new;
+            l[g] = l[g] * alpha + pr;
+#pragma unroll
+            for (int e = 0; e < N; ++e) acc[g][e] = fmaf(pr, vf[e], acc[g][e] * alpha);
+        }
+    }
+
+    // merge the TPW lane groups of the wave
+#pragma unroll
+    for (int o = LPR; o < WAVE; o <<= 1) {
+#pragma unroll
+        for (int g = 0; g < GMAX; ++g) {
+            const float mo = __shfl_xor(m[g], o);
+            const float lo = __shfl_xor(l[g], o);
+            const float mn = fmaxf(m[g], mo);
+            const float a = exp2f(m[g] - mn), b = exp2f(mo - mn);
+            l[g] = l[g] * a + lo * b;
+#pragma unroll
+            for (int e = 0; e < N; ++e) {
+                const float ao = __shfl_xor(acc[g][e], o);
+                acc[g][e] = acc[g][e] * a + ao * b;
+            }
+            m[g] = mn;
+        }
+    }
+
+    // merge the waves through LDS
+    __shared__ float sm_m[NW][GMAX];
+    __shared__ float sm_l[NW][GMAX];
+    __shared__ float sm_acc[NW][GMAX][D];
+    if (sub == 0) {
+#pragma unroll
+        for (int g = 0; g < GMAX; ++g) {
+            if (lr == 0) { sm_m[w][g] = m[g]; sm_l[w][g] = l[g]; }
+#pragma unroll
+            for (int e = 0; e < N; ++e) sm_acc[w][g][lr * N + e] = acc[g][e];
+        }
+    }
+    __syncthreads();
+
+    const float vs = p.v_scale ? p.v_scale[kvh] : 1.f;
+    for (int i = tid; i < gn * D; i += blockDim.x) {
+        const int g = i / D, dd = i % D;
+        float mx = sm_m[0][g];
+#pragma unroll
+        for (int ww = 1; ww < NW; ++ww) mx = fmaxf(mx, sm_m[ww][g]);
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < NW; ++ww) {
+            const float f = exp2f(sm_m[ww][g] - mx);
+            num = fmaf(f, sm_acc[ww][g][dd], num);
+            den = fmaf(f, sm_l[ww][g], den);
+        }
+        const int head = head0 + g;
+        if (p.num_parts == 1) {
+            store_elem<Q_T>((Q_T*)p.out + (row * p.hq + head) * D + dd, den > 0.f ? vs * num / den : 0.f);
+        } else {
+            const int64_t slot = (row * p.hq + head) * p.num_parts + part;
+            p.ws_acc[slot * D + dd] = num;
+            if (dd == 0) { p.ws_ml[slot * 2] = mx; p.ws_ml[slot * 2 + 1] = den; }
+        }
+    }
+}
+
+// Split-K merge: out = sum_p 2^(m_p - M) acc_p / sum_p 2^(m_p - M) l_p, M = max_p m_p.
+// One workgroup per (row, head); only the partitions that hold tokens are read.
+template <typename Q_T>
+__global__ void __launch_bounds__(256)
+split_reduce_kernel(Q_T* __restrict__ out, const float* __restrict__ ws_acc,
+                    const float* __restrict__ ws_ml, const int32_t* __restrict__ context_lens,
+                    const int32_t* __restrict__ cu_q_lens, int num_seqs, int hq, int group, int d,
+                    int partition_size, int num_parts, const float* __restrict__ v_scale) {
+    const int64_t row = blockIdx.x;
+    const int head = blockIdx.y;
+    int seq, len;
+    row_info(row, cu_q_lens, context_lens, num_seqs, seq, len);
+    const int np = min(num_parts, (len + partition_size - 1) / partition_size);
+    const int64_t slot0 = (row * hq + head) * num_parts;
+    float mx = NEG_BIG;
+    for (int pi = 0; pi < np; ++pi) mx = fmaxf(mx, ws_ml[(slot0 + pi) * 2]);
+    float den = 0.f;
+    for (int pi = 0; pi < np; ++pi)
+        den = fmaf(exp2f(ws_ml[(slot0 + pi) * 2] - mx), ws_ml[(slot0 + pi) * 2 + 1], den);
+    const float vs = v_scale ? v_scale[head / group] : 1.f;
+    const float inv = den > 0.f ? vs / den : 0.f;
+    for (int dd = threadIdx.x; dd < d; dd += blockDim.x) {
+        float num = 0.f;
+        for (int pi = 0; pi < np; ++pi)
+            num = fmaf(exp2f(ws_ml[(slot0 + pi) * 2] - mx), ws_acc[(slot0 + pi) * d + dd], num);
+        store_elem<Q_T>(out + (row * hq + head) * d + dd, num * inv);
+    }
+}
+
+int launch_split_reduce(const DecodeArgs& a) {
+    dim3 grid((unsigned)a.rows, (unsigned)a.hq);
+    const int threads = a.d <= 64 ? 64 : (a.d <= 128 ? 128 : 256);
+    const int group = a.hq / a.hkv;
+    if (a.q_dtype == AICOMP_KV_F32)
+        hipLaunchKernelGGL(split_reduce_kernel<float>, grid, dim3(threads), 0, a.stream,
+                           (float*)a.out, a.ws.acc, a.ws.ml, a.context_lens, a.cu_q_lens,
+                           a.num_seqs, a.hq, group, a.d, a.partition_size, a.num_parts, a.v_scale);
+    else
+        hipLaunchKernelGGL(split_reduce_kernel<bf16_t>, grid, dim3(threads), 0, a.stream,
+                           (bf16_t*)a.out, a.ws.acc, a.ws.ml, a.context_lens, a.cu_q_lens,
+                           a.num_seqs, a.hq, group, a.d, a.partition_size, a.num_parts, a.v_scale);
+    AICOMP_HIP_LAUNCH_CHECK();
+    return AICOMP_KV_OK;
+}
+
+template <typename KV_T, typename Q_T, int D>
+static int launch_generic_d(const DecodeArgs& a, const GenericParams& p) {
+    const int group = a.hq / a.hkv;
+    if (group <= 4) {
+        dim3 grid((unsigned)a.rows, (unsigned)a.hkv, (unsigned)a.num_parts);
+        hipLaunchKernelGGL((paged_attn_generic_kernel<KV_T, Q_T, D, 4>), grid, dim3(256), 0,
+                           a.stream, p);
+    } else {
+        const int gpk = (group + 7) / 8;
+        dim3 grid((unsigned)a.rows, (unsigned)(a.hkv * gpk), (unsigned)a.num_parts);
+        hipLaunchKernelGGL((paged_attn_generic_kernel<KV_T, Q_T, D, 8>), grid, dim3(256), 0,
+                           a.stream, p);
+    }
+    AICOMP_HIP_LAUNCH_CHECK();
+    return AICOMP_KV_OK;
+}
+
+template <typename KV_T, typename Q_T>
+static int launch_generic_t(const DecodeArgs& a, const GenericParams& p) {
+    switch (a.d) {
+        case 64: return launch_generic_d<KV_T, Q_T, 64>(a, p);
+        case 128: return launch_generic_d<KV_T, Q_T, 128>(a, p);
+        case 256: return launch_generic_d<KV_T, Q_T, 256>(a, p);
+        default:
+            set_error("paged attention: head_dim %d not supported (64, 128, 256)", a.d);
+            return AICOMP_KV_EUNSUPPORTED;
+    }
+}
+
+int launch_decode_generic(const DecodeArgs& a) {
+    if (a.rows == 0) return AICOMP_KV_OK;
+    AICOMP_REQUIRE(a.rows < (1ll << 31) && a.num_parts <= 65535 && a.hkv * ((a.hq / a.hkv + 7) / 8) <= 65535, AICOMP_KV_EINVAL,
+                   "paged attention: grid too large");
+    GenericParams p;
+    p.out = a.out; p.query = a.query; p.k_pool = a.k_pool; p.v_pool = a.v_pool;
+    p.block_table = a.block_table; p.block_table_stride = a.block_table_stride;
+    p.context_lens = a.context_lens; p.cu_q_lens = a.cu_q_lens; p.num_seqs = a.num_seqs;
+    p.hq = a.hq; p.hkv = a.hkv; p.group = a.hq / a.hkv; p.bs = a.bs; p.num_blocks = a.num_blocks;
+    p.qk_mul = a.scale * LOG2E;
+    p.k_scale = a.k_scale; p.v_scale = a.v_scale;
+    p.partition_size = a.partition_size; p.num_parts = a.num_parts;
+    p.ws_acc = a.ws.acc; p.ws_ml = a.ws.ml;
+    int rc;
+    if (a.kv_dtype == AICOMP_KV_F32 && a.q_dtype == AICOMP_KV_F32)
+        rc = launch_generic_t<float, float>(a, p);
+    else if (a.kv_dtype == AICOMP_KV_BF16 && a.q_dtype == AICOMP_KV_BF16)
+        rc = launch_generic_t<bf16_t, bf16_t>(a, p);
+    else if (a.kv_dtype == AICOMP_KV_FP8_E4M3 && a.q_dtype == AICOMP_KV_BF16)
+        rc = launch_generic_t<fp8_t, bf16_t>(a, p);
+    else {
+        set_error("paged attention: unsupported type pair (query %d, pool %d); supported: "
+                  "f32/f32, bf16/bf16, bf16/fp8", a.q_dtype, a.kv_dtype);
+        return AICOMP_KV_EUNSUPPORTED;
+    }
+    if (rc != AICOMP_KV_OK) return rc;
+    if (a.num_parts > 1) return launch_split_reduce(a);
+    return AICOMP_KV_OK;
+}
+
+}  // namespace aicomp

@@ -1,0 +1,200 @@
+"""Tensor-level wrappers of the C ABI: the three native ops of the path.
+
+``kv_append``, ``paged_decode_attn`` and ``paged_prefill_attn`` take torch
+tensors on a ROCm device, check them the way a ``TORCH_CHECK`` would
+(``RuntimeError`` on dtype / shape / contiguity / device mismatch), and pass
+raw device pointers plus the current HIP stream to libaicomp_kv.so.  torch is
+used for device memory and streams only.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_DT = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float8_e4m3fn: _lib.FP8_E4M3}
+
+
+def _dt(t: torch.Tensor, what: str) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise RuntimeError(f"{what}: unsupported dtype {t.dtype} (float32, bfloat16, float8_e4m3fn)")
+
+
+def _req(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _dev(t: torch.Tensor, ref: torch.Tensor, what: str) -> None:
+    _req(t.device == ref.device, f"{what} is on {t.device}, expected {ref.device}")
+
+
+def _stream(t: torch.Tensor) -> int:
+    _req(t.is_cuda, "tensors must live on a ROCm device (there is no CPU path)")
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _check_pools(k_pool: torch.Tensor, v_pool: torch.Tensor) -> Tuple[int, int, int, int]:
+    _req(k_pool.dim() == 4 and v_pool.shape == k_pool.shape,
+         f"pools must both be [num_blocks, Hkv, BS, D]; got {tuple(k_pool.shape)} and {tuple(v_pool.shape)}")
+    _req(k_pool.dtype == v_pool.dtype, "k_pool and v_pool dtypes differ")
+    _req(k_pool.is_contiguous() and v_pool.is_contiguous(), "pools must be contiguous")
+    _dev(v_pool, k_pool, "v_pool")
+    return tuple(k_pool.shape)  # type: ignore[return-value]
+
+
+def _check_scales(k_scale, v_scale, pool: torch.Tensor, hkv: int):
+    if pool.dtype == torch.float8_e4m3fn:
+        _req(k_scale is not None and v_scale is not None, "an fp8 pool needs k_scale and v_scale")
+        for s, n in ((k_scale, "k_scale"), (v_scale, "v_scale")):
+            _req(s.dtype == torch.float32 and s.is_contiguous() and s.numel() == hkv,
+                 f"{n} must be a contiguous float32 tensor of {hkv} elements")
+            _dev(s, pool, n)
+        return k_scale, v_scale
+    return None, None
+
+
+def kv_append(key: torch.Tensor, value: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+              slot_mapping: torch.Tensor, k_scale: Optional[torch.Tensor] = None,
+              v_scale: Optional[torch.Tensor] = None) -> None:
+    """Scatter ``key/value [T, Hkv, D]`` into the pools at ``slot_mapping [T]`` (int64).
+
+    In place on the pools, on the current stream.  Same dtype in and out is a
+    raw copy; a float8_e4m3fn pool quantises with the per-KV-head scales.
+    """
+    lib = _lib.load()
+    nb, hkv, bs, d = _check_pools(k_pool, v_pool)
+    _req(key.dim() == 3 and key.shape == value.shape and key.dtype == value.dtype,
+         f"key/value must both be [T, Hkv, D]; got {tuple(key.shape)} and {tuple(value.shape)}")
+    _req(key.shape[1] == hkv and key.shape[2] == d,
+         f"key is [T, {key.shape[1]}, {key.shape[2]}] but the pool holds [{hkv}, {d}] rows")
+    _req(slot_mapping.dtype == torch.int64 and slot_mapping.dim() == 1
+         and slot_mapping.numel() == key.shape[0] and slot_mapping.is_contiguous(),
+         "slot_mapping must be a contiguous int64 vector with one entry per row")
+    for t, n in ((value, "value"), (k_pool, "k_pool"), (slot_mapping, "slot_mapping")):
+        _dev(t, key, n)
+    ks, vs = (None, None) if key.dtype == k_pool.dtype else _check_scales(k_scale, v_scale, k_pool, hkv)
+    if key.stride(2) != 1 or key.stride() != value.stride():
+        key, value = key.contiguous(), value.contiguous()
+    rc = lib.aicomp_kv_append(key.data_ptr(), value.data_ptr(), key.stride(0), key.stride(1),
+                              k_pool.data_ptr(), v_pool.data_ptr(), slot_mapping.data_ptr(),
+                              key.shape[0], hkv, d, bs, nb, _dt(key, "key"), _dt(k_pool, "pool"),
+                              _ptr(ks), _ptr(vs), _stream(key))
+    _lib.check(rc, lib)
+
+
+# split-K scratch, one growing buffer per (device, stream)
+_workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def _workspace(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
+    if nbytes == 0:
+        return None
+    key = (device.index or 0, torch.cuda.current_stream(device).cuda_stream)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def decode_partition_size(batch: int, hq: int, hkv: int, d: int, bs: int, max_blocks: int,
+                          q_dtype: torch.dtype, kv_dtype: torch.dtype) -> int:
+    lib = _lib.load()
+    return lib.aicomp_paged_decode_partition_size(batch, hq, hkv, d, bs, max_blocks,
+                                                  _DT[q_dtype], _DT[kv_dtype])
+
+
+def paged_decode_attn(out: torch.Tensor, query: torch.Tensor, k_pool: torch.Tensor,
+                      v_pool: torch.Tensor, block_table: torch.Tensor,
+                      context_lens: torch.Tensor, scale: float,
+                      k_scale: Optional[torch.Tensor] = None,
+                      v_scale: Optional[torch.Tensor] = None, partition_size: int = 0,
+                      workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out[b, h] = softmax(q[b, h] . K_b^T * scale) V_b`` over the paged context.
+
+    ``out``/``query`` ``[B, Hq, D]``; ``block_table [B, max_blocks]`` int32;
+    ``context_lens [B]`` int32.  In place on ``out``, on the current stream.
+    """
+    lib = _lib.load()
+    nb, hkv, bs, d = _check_pools(k_pool, v_pool)
+    _req(query.dim() == 3 and out.shape == query.shape and out.dtype == query.dtype,
+         f"out/query must both be [B, Hq, D]; got {tuple(out.shape)} and {tuple(query.shape)}")
+    B, hq, dq = query.shape
+    _req(dq == d, f"query head_dim {dq} != pool head_dim {d}")
+    _req(query.is_contiguous() and out.is_contiguous(), "query and out must be contiguous")
+    _req(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] == B
+         and block_table.stride(1) == 1, "block_table must be int32 [B, max_blocks], rows contiguous")
+    _req(context_lens.dtype == torch.int32 and context_lens.numel() == B
+         and context_lens.is_contiguous(), "context_lens must be contiguous int32 [B]")
+    for t, n in ((out, "out"), (k_pool, "k_pool"), (block_table, "block_table"),
+                 (context_lens, "context_lens")):
+        _dev(t, query, n)
+    ks, vs = _check_scales(k_scale, v_scale, k_pool, hkv)
+    qd, kd = _dt(query, "query"), _dt(k_pool, "pool")
+    need = lib.aicomp_paged_decode_workspace_bytes(B, hq, hkv, d, bs, block_table.shape[1], qd, kd,
+                                                   partition_size)
+    if workspace is None:
+        workspace = _workspace(query.device, need)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    rc = lib.aicomp_paged_decode_attn(out.data_ptr(), query.data_ptr(), k_pool.data_ptr(),
+                                      v_pool.data_ptr(), block_table.data_ptr(),
+                                      block_table.stride(0), context_lens.data_ptr(), B, hq, hkv, d,
+                                      bs, block_table.shape[1], nb, float(scale), qd, kd,
+                                      _ptr(ks), _ptr(vs), partition_size, _ptr(workspace),
+                                      ws_bytes, _stream(query))
+    _lib.check(rc, lib)
+    return out
+
+
+def paged_prefill_attn(out: torch.Tensor, query: torch.Tensor, k_pool: torch.Tensor,
+                       v_pool: torch.Tensor, block_table: torch.Tensor,
+                       context_lens: torch.Tensor, cu_q_lens: torch.Tensor, scale: float,
+                       max_q_len: Optional[int] = None,
+                       k_scale: Optional[torch.Tensor] = None,
+                       v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal attention of concatenated chunks ``query [T, Hq, D]`` over the pool.
+
+    Chunk s owns rows ``cu_q_lens[s]:cu_q_lens[s+1]``; its context of
+    ``context_lens[s]`` tokens (chunk included) must already be in the pool.
+    ``max_q_len`` is the host-side bound on the chunk lengths; when omitted it
+    is read back from ``cu_q_lens`` (a device synchronisation).
+    """
+    lib = _lib.load()
+    nb, hkv, bs, d = _check_pools(k_pool, v_pool)
+    _req(query.dim() == 3 and out.shape == query.shape and out.dtype == query.dtype,
+         f"out/query must both be [T, Hq, D]; got {tuple(out.shape)} and {tuple(query.shape)}")
+    T, hq, dq = query.shape
+    _req(dq == d, f"query head_dim {dq} != pool head_dim {d}")
+    _req(query.is_contiguous() and out.is_contiguous(), "query and out must be contiguous")
+    S = context_lens.numel()
+    _req(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] == S
+         and block_table.stride(1) == 1, "block_table must be int32 [S, max_blocks], rows contiguous")
+    _req(context_lens.dtype == torch.int32 and context_lens.is_contiguous(),
+         "context_lens must be contiguous int32 [S]")
+    _req(cu_q_lens.dtype == torch.int32 and cu_q_lens.numel() == S + 1 and cu_q_lens.is_contiguous(),
+         "cu_q_lens must be contiguous int32 [S+1]")
+    for t, n in ((out, "out"), (k_pool, "k_pool"), (block_table, "block_table"),
+                 (context_lens, "context_lens"), (cu_q_lens, "cu_q_lens")):
+        _dev(t, query, n)
+    ks, vs = _check_scales(k_scale, v_scale, k_pool, hkv)
+    if max_q_len is None:
+        cu = cu_q_lens.cpu()
+        max_q_len = int((cu[1:] - cu[:-1]).max()) if S else 0
+    rc = lib.aicomp_paged_prefill_attn(out.data_ptr(), query.data_ptr(), k_pool.data_ptr(),
+                                       v_pool.data_ptr(), block_table.data_ptr(),
+                                       block_table.stride(0), context_lens.data_ptr(),
+                                       cu_q_lens.data_ptr(), S, T, int(max_q_len), hq, hkv, d, bs,
+                                       block_table.shape[1], nb, float(scale),
+                                       _dt(query, "query"), _dt(k_pool, "pool"), _ptr(ks), _ptr(vs),
+                                       _stream(query))
+    _lib.check(rc, lib)
+    return out

@@ -1,0 +1,146 @@
+/*
+ * aicomp_kv.h - C ABI of the MI355X (gfx950) paged KV-cache attention library.
+ *
+ * This is the whole drop-in boundary: plain pointers, sizes and a HIP stream
+ * handle.  Every pointer except `stream` is DEVICE memory owned by the caller
+ * and borrowed for the duration of the call; nothing is allocated, freed or
+ * synchronised inside the library.  All work is enqueued on `stream`
+ * (a hipStream_t passed as void*; NULL = the default stream).
+ *
+ * The operator being replaced is the reference's
+ *   CachedScaledDotProductAttention.forward     opt_prime/opt_prime/kv_cache.py:340-415
+ *   KVCacheManager.update                       opt_prime/opt_prime/kv_cache.py:112-170
+ * which run, per transformer layer and per step, (1) a slice-assign append of
+ * the new K/V rows, (2) a .contiguous() copy of the whole prefix and (3)
+ * torch's scaled_dot_product_attention.  The entry points below are those
+ * three steps on a paged pool, with (2) removed.
+ *
+ * Pool layout (both pools):  [num_blocks, num_kv_heads, block_size, head_dim],
+ * contiguous.  Token t of sequence s lives at slot
+ *   block_table[s][t / block_size] * block_size + t % block_size.
+ * Heads in the pool are KV heads; query head h reads KV head h / (Hq / Hkv),
+ * the order HF Llama's repeat_kv produces (compiler_fx/modeling_llama.py:268-277).
+ *
+ * Return value: 0 on success, otherwise one of the AICOMP_KV_E* codes; the
+ * message of the last failure on the calling thread is aicomp_kv_last_error().
+ */
+#ifndef AICOMP_KV_H
+#define AICOMP_KV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AICOMP_KV_OK            0
+#define AICOMP_KV_EINVAL        1   /* bad shape / dtype / null pointer / size   */
+#define AICOMP_KV_EUNSUPPORTED  2   /* valid request the kernels do not cover    */
+#define AICOMP_KV_EHIP          3   /* a HIP runtime call failed                 */
+#define AICOMP_KV_EWORKSPACE    4   /* workspace missing or too small            */
+
+/* element types */
+#define AICOMP_KV_F32       0
+#define AICOMP_KV_BF16      1
+#define AICOMP_KV_FP8_E4M3  2       /* OCP e4m3 ("e4m3fn"), max finite 448       */
+
+/* Library version (major*10000 + minor*100 + patch). */
+int aicomp_kv_version(void);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* aicomp_kv_last_error(void);
+
+/*
+ * KV append: scatter T new rows into the pools by slot_mapping.
+ * Replaces  key_cache[:, :, position:end_position, :] = new_k   (kv_cache.py:159-160)
+ * and       self.cache_k[:, :, self.cache_pos:end_pos, :] = key (kv_cache.py:387-388).
+ *
+ *   key, value     [T, Hkv, D] of in_dtype; element (t,h,d) is at
+ *                  t*kv_token_stride + h*kv_head_stride + d  (strides in elements)
+ *   k_pool, v_pool pools of pool_dtype
+ *   slot_mapping   [T] int64; slot < 0 skips the row; slots must be distinct
+ *   in_dtype == pool_dtype                  raw copy, bit-exact
+ *   in_dtype f32/bf16, pool_dtype FP8_E4M3  code = e4m3_rne(clamp(x / scale[h], +-448)),
+ *                                           k_scale / v_scale [Hkv] float, required
+ */
+int aicomp_kv_append(const void* key, const void* value,
+                     int64_t kv_token_stride, int64_t kv_head_stride,
+                     void* k_pool, void* v_pool, const int64_t* slot_mapping,
+                     int64_t num_tokens, int num_kv_heads, int head_dim,
+                     int block_size, int64_t num_blocks,
+                     int in_dtype, int pool_dtype,
+                     const float* k_scale, const float* v_scale,
+                     void* stream);
+
+/*
+ * Paged decode attention: one query token per sequence, no mask.
+ * Replaces the decode branch  F.scaled_dot_product_attention(query, full_key,
+ * full_value, attn_mask=None, is_causal=False)   (kv_cache.py:397-403)
+ * including the .contiguous() prefix copies it is fed from (kv_cache.py:391-392).
+ *
+ *   out, query      [B, Hq, D] of q_dtype, contiguous
+ *   block_table     [B, max_blocks_per_seq] int32, row stride block_table_stride
+ *   context_lens    [B] int32, tokens to attend to (0 -> the output row is zero)
+ *   scale           softmax scale (the reference's default is 1/sqrt(D))
+ *   kv_dtype FP8    k_scale / v_scale [Hkv] float dequantisation factors, fused
+ *                   into the loads
+ *   partition_size  split-K (flash-decoding) tokens per partition; 0 = choose
+ *                   from the shape; a multiple of block_size otherwise.  With
+ *                   more than one partition a second kernel merges the
+ *                   partial (max, sum, output) triples.
+ *   workspace       device scratch of at least
+ *                   aicomp_paged_decode_workspace_bytes(...) bytes (may be NULL
+ *                   when that returns 0)
+ */
+int aicomp_paged_decode_attn(void* out, const void* query,
+                             const void* k_pool, const void* v_pool,
+                             const int32_t* block_table, int64_t block_table_stride,
+                             const int32_t* context_lens,
+                             int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                             int block_size, int max_blocks_per_seq, int64_t num_blocks,
+                             float scale, int q_dtype, int kv_dtype,
+                             const float* k_scale, const float* v_scale,
+                             int partition_size,
+                             void* workspace, size_t workspace_bytes,
+                             void* stream);
+
+size_t aicomp_paged_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads,
+                                           int head_dim, int block_size,
+                                           int max_blocks_per_seq, int q_dtype, int kv_dtype,
+                                           int partition_size);
+
+/* The partition size the library would pick for partition_size == 0. */
+int aicomp_paged_decode_partition_size(int batch, int num_q_heads, int num_kv_heads,
+                                       int head_dim, int block_size,
+                                       int max_blocks_per_seq, int q_dtype, int kv_dtype);
+
+/*
+ * Chunked-prefill causal attention over the paged pool (MFMA bf16).
+ * Replaces the prefill branch  F.scaled_dot_product_attention(query, full_key,
+ * full_value, attn_mask=None, is_causal=True)   (kv_cache.py:404-415).
+ * The chunk's own K/V rows must already be in the pool (append first).
+ *
+ *   out, query     [T, Hq, D] bf16, rows of sequence s are cu_q_lens[s]..cu_q_lens[s+1]
+ *   context_lens   [S] int32: prior context + chunk length
+ *   cu_q_lens      [S+1] int32 prefix sums of the chunk lengths
+ *   max_q_len      host-side upper bound of the chunk lengths (sizes the grid)
+ * Mask: query i of a chunk with prior context P sees keys j <= P + i
+ * (bottom-right aligned; P == 0 is the reference's is_causal=True, a chunk of
+ * one token is the reference's decode).
+ */
+int aicomp_paged_prefill_attn(void* out, const void* query,
+                              const void* k_pool, const void* v_pool,
+                              const int32_t* block_table, int64_t block_table_stride,
+                              const int32_t* context_lens, const int32_t* cu_q_lens,
+                              int num_seqs, int64_t total_q, int max_q_len,
+                              int num_q_heads, int num_kv_heads, int head_dim,
+                              int block_size, int max_blocks_per_seq, int64_t num_blocks,
+                              float scale, int q_dtype, int kv_dtype,
+                              const float* k_scale, const float* v_scale,
+                              void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AICOMP_KV_H */

@@ -1,0 +1,194 @@
+"""Paged decode attention through the C ABI vs the float64 oracle."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from aicomp_amd import ops, workloads
+from oracle import paged_kv_oracle as orc
+from helpers import NAME, assert_close_attn, raw, to_f64
+
+pytestmark = pytest.mark.gpu
+
+# bf16 tolerance of the benchmark definition: max-abs 1e-2 or relative 2e-2 vs fp32/64
+BF16_ATOL, BF16_RTOL = 1e-2, 2e-2
+F32_ATOL = 1e-5
+
+
+def oracle_decode(w, ctx=None):
+    ks = None if w.k_scale is None else w.k_scale.cpu().numpy()
+    vs = None if w.v_scale is None else w.v_scale.cpu().numpy()
+    return orc.paged_decode_attn(raw(w.query), raw(w.k_pool), raw(w.v_pool),
+                                 w.block_table.cpu().numpy(),
+                                 (w.context_lens.cpu().numpy() if ctx is None else ctx), w.scale,
+                                 q_dtype=NAME[w.query.dtype], kv_dtype=NAME[w.k_pool.dtype],
+                                 k_scale=ks, v_scale=vs)
+
+
+def run_decode(w, partition_size=0, ctx=None):
+    out = torch.full_like(w.query, float("nan"))
+    ops.paged_decode_attn(out, w.query, w.k_pool, w.v_pool, w.block_table,
+                          w.context_lens if ctx is None else ctx, w.scale,
+                          k_scale=w.k_scale, v_scale=w.v_scale, partition_size=partition_size)
+    torch.cuda.synchronize()
+    return out
+
+
+def small(name, **kw):
+    s = workloads.SHAPES[name]
+    return workloads.Shape(**{**s.__dict__, **kw})
+
+
+def test_config1_fp32_anchor(device):
+    """batch 4, 32/8 heads, D 64, L in [64,512], pool of 256 blocks: <= 1e-5 abs."""
+    w = workloads.make_workload("decode_fp32_small", device=device)
+    want = oracle_decode(w)
+    for ps in (0, 64, 16 * 64):
+        got = to_f64(run_decode(w, ps))
+        assert np.abs(got - want).max() <= F32_ATOL, ps
+
+
+@pytest.mark.parametrize("ps", [0, 256, 1024, 8192])
+def test_config2_shape_reduced_batch(device, ps):
+    """Llama-3-8B decode shape, batch cut to 6 so the oracle runs in seconds."""
+    w = workloads.make_workload("x", device=device, shape=small("llama3_8b_decode", batch=6))
+    ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping)
+    want = oracle_decode(w)
+    got = to_f64(run_decode(w, ps))
+    assert_close_attn(got, want, BF16_ATOL, BF16_RTOL, f"partition {ps}")
+
+
+@pytest.mark.parametrize("hq,hkv,d,bs,dtype", [
+    (8, 8, 64, 16, torch.bfloat16),       # MHA
+    (8, 1, 128, 16, torch.bfloat16),      # MQA, group 8
+    (12, 2, 128, 16, torch.bfloat16),     # group 6
+    (32, 2, 128, 16, torch.bfloat16),     # group 16
+    (6, 2, 256, 8, torch.bfloat16),
+    (4, 2, 128, 32, torch.float32),
+    (4, 4, 64, 1, torch.float32),         # block size 1
+])
+def test_decode_shapes(device, hq, hkv, d, bs, dtype):
+    sh = workloads.Shape("t", 5, hq, hkv, d, block_size=bs, q_dtype=dtype, kv_dtype=dtype,
+                         ctx_lo=1, ctx_hi=700)
+    w = workloads.make_workload("t", device=device, seed=3, shape=sh)
+    want = oracle_decode(w)
+    for ps in (0, 32 * bs if bs > 1 else 64):
+        got = to_f64(run_decode(w, ps))
+        if dtype == torch.float32:
+            assert np.abs(got - want).max() <= F32_ATOL
+        else:
+            assert_close_attn(got, want, BF16_ATOL, BF16_RTOL, f"{hq}/{hkv} D{d} BS{bs} ps{ps}")
+
+
+def test_decode_edge_lengths(device):
+    """Context lengths 0, 1, block boundaries, and NaN/Inf poison beyond the context."""
+    sh = workloads.Shape("t", 8, 8, 2, 128, ctx_lo=300, ctx_hi=300)
+    w = workloads.make_workload("t", device=device, seed=4, shape=sh)
+    ctx = torch.tensor([0, 1, 15, 16, 17, 255, 256, 301], dtype=torch.int32, device=device)
+    bs = 16
+    # poison every slot at or beyond each sequence's context, and every unused block
+    used = torch.zeros(w.k_pool.shape[0] * bs, dtype=torch.bool, device=device)
+    for b, L in enumerate(ctx.tolist()):
+        t = torch.arange(L, device=device)
+        used[w.block_table[b, t // bs].long() * bs + t % bs] = True
+    kf = w.k_pool.permute(0, 2, 1, 3).reshape(-1, 2, 128).clone()
+    vf = w.v_pool.permute(0, 2, 1, 3).reshape(-1, 2, 128).clone()
+    kf[~used] = float("nan")
+    vf[~used] = float("inf")
+    w.k_pool = kf.reshape(-1, bs, 2, 128).permute(0, 2, 1, 3).contiguous()
+    w.v_pool = vf.reshape(-1, bs, 2, 128).permute(0, 2, 1, 3).contiguous()
+    kclean = torch.nan_to_num(w.k_pool.float(), nan=0.0).to(torch.bfloat16)
+    vclean = torch.nan_to_num(w.v_pool.float(), posinf=0.0).to(torch.bfloat16)
+    want = orc.paged_decode_attn(raw(w.query), raw(kclean), raw(vclean), w.block_table.cpu().numpy(),
+                                 ctx.cpu().numpy(), w.scale, "bf16", "bf16")
+    for ps in (0, 64, 512):
+        got = to_f64(run_decode(w, ps, ctx=ctx))
+        assert_close_attn(got, want, BF16_ATOL, BF16_RTOL, f"ps {ps}")
+        assert np.array_equal(got[0], np.zeros_like(got[0]))
+        # L == 1: the output is exactly the V row (bf16 in, bf16 out)
+        v_row = to_f64(vclean[w.block_table[1, 0].long(), :, 0, :])       # [Hkv, D]
+        assert np.array_equal(got[1], np.repeat(v_row, 4, axis=0))
+
+
+def test_decode_invariants(device):
+    sh = workloads.Shape("t", 4, 8, 2, 128, ctx_lo=200, ctx_hi=900, kv_std=0.5)
+    w = workloads.make_workload("t", device=device, seed=5, shape=sh)
+    base = run_decode(w, 256)
+    # split sizes agree to fp32 round-off (outputs are bf16: allow one ulp)
+    for ps in (0, 128, 512, 2048):
+        o = run_decode(w, ps)
+        assert (o.float() - base.float()).abs().max() <= 2 ** -8 * base.float().abs().max()
+    # moving blocks with the table updated: bit-identical for a fixed partitioning
+    nb = w.k_pool.shape[0]
+    perm = torch.randperm(nb, device=device)
+    kp2, vp2 = torch.empty_like(w.k_pool), torch.empty_like(w.v_pool)
+    kp2[perm] = w.k_pool
+    vp2[perm] = w.v_pool
+    w2 = workloads.Workload(**{**w.__dict__, "k_pool": kp2, "v_pool": vp2,
+                               "block_table": perm[w.block_table.long()].to(torch.int32)})
+    assert torch.equal(run_decode(w2, 256).view(torch.int16), base.view(torch.int16))
+    # same query in all heads of a group -> same output
+    q = w.query.clone()
+    q[:, 1:4] = q[:, 0:1]
+    w3 = workloads.Workload(**{**w.__dict__, "query": q})
+    o = run_decode(w3, 256)
+    assert torch.equal(o[:, 1].view(torch.int16), o[:, 0].view(torch.int16))
+    # all keys equal -> output = mean of V
+    w4 = workloads.Workload(**{**w.__dict__, "k_pool": torch.ones_like(w.k_pool)})
+    o = to_f64(run_decode(w4, 256))
+    for b, L in enumerate(w.ctx_list):
+        v = orc.bf16_bits_to_f32(orc.gather_context(raw(w.v_pool), w.block_table[b].cpu().numpy(), L))
+        assert np.abs(o[b] - np.repeat(v.mean(axis=0), 4, axis=0)).max() <= 1e-2
+    # a huge common score offset changes nothing (online-softmax max handling)
+    w5 = workloads.Workload(**{**w.__dict__, "k_pool": (w.k_pool.float() * 0 + 3.0).to(torch.bfloat16),
+                               "query": (w.query.float() * 0 + 8.0).to(torch.bfloat16)})
+    o5 = to_f64(run_decode(w5, 256))       # every score = 8*3*128*scale ~ 271
+    assert np.isfinite(o5).all()
+    assert np.abs(o5 - o).max() <= 1e-2
+
+
+def test_decode_errors(device):
+    sh = workloads.Shape("t", 2, 8, 2, 128, ctx_lo=20, ctx_hi=40)
+    w = workloads.make_workload("t", device=device, shape=sh)
+    out = torch.empty_like(w.query)
+    with pytest.raises(RuntimeError):
+        ops.paged_decode_attn(out, w.query, w.k_pool, w.v_pool, w.block_table.long(), w.context_lens, 1.0)
+    with pytest.raises(RuntimeError):
+        ops.paged_decode_attn(out, w.query, w.k_pool, w.v_pool.float(), w.block_table, w.context_lens, 1.0)
+    with pytest.raises(RuntimeError):
+        ops.paged_decode_attn(out[:, :6], w.query[:, :6], w.k_pool, w.v_pool, w.block_table, w.context_lens, 1.0)
+    with pytest.raises(RuntimeError):
+        ops.paged_decode_attn(out, w.query, w.k_pool, w.v_pool, w.block_table, w.context_lens, 1.0,
+                              partition_size=24)
+    with pytest.raises(RuntimeError):
+        ops.paged_decode_attn(out.cpu(), w.query.cpu(), w.k_pool.cpu(), w.v_pool.cpu(),
+                              w.block_table.cpu(), w.context_lens.cpu(), 1.0)
+    q96 = torch.zeros(2, 8, 96, dtype=torch.bfloat16, device=device)
+    p96 = torch.zeros(4, 2, 16, 96, dtype=torch.bfloat16, device=device)
+    with pytest.raises(RuntimeError):
+        ops.paged_decode_attn(torch.empty_like(q96), q96, p96, p96, w.block_table, w.context_lens, 1.0)
+
+
+def test_fp8_decode_vs_dequantised_oracle(device):
+    """fp8 e4m3 KV with per-head scales, group 8: within the bf16 tolerance of the
+    oracle run on the dequantised values; wider stated bound vs unquantised."""
+    w = workloads.make_workload("x", device=device, shape=small("llama3_70b_decode_fp8", batch=4))
+    ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping, w.k_scale, w.v_scale)
+    want = oracle_decode(w)
+    for ps in (0, 512):
+        got = to_f64(run_decode(w, ps))
+        assert_close_attn(got, want, BF16_ATOL, BF16_RTOL, f"fp8 ps {ps}")
+
+
+def test_config3_long_context_split(device):
+    """Long-context skewed batch (log-normal, sigma 1.0, clip [256,32768]), batch cut to 4."""
+    w = workloads.make_workload("x", device=device, seed=0,
+                                shape=small("long_context_skewed", batch=4))
+    ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping)
+    want = oracle_decode(w)
+    got = to_f64(run_decode(w, 0))
+    assert_close_attn(got, want, BF16_ATOL, BF16_RTOL, "auto split")
+    got1 = to_f64(run_decode(w, w.block_table.shape[1] * 16))      # one partition
+    assert_close_attn(got1, want, BF16_ATOL, BF16_RTOL, "unsplit")
+    assert np.abs(got - got1).max() <= 2 ** -7 * np.abs(got1).max()
