@@ -1,5 +1,357 @@
+// Paged decode attention on gfx950 matrix cores: the hot kernel of the path.
+//
+// Replaces  F.scaled_dot_product_attention(query, full_key, full_value,
+//           attn_mask=None, is_causal=False)      opt_prime/opt_prime/kv_cache.py:397-403
+// and the two .contiguous() prefix copies that feed it (kv_cache.py:391-392):
+// K and V are read once, in place, through the block table.
+//
+// Shape covered: head_dim 128, block_size 16, bf16 queries, bf16 or fp8-e4m3
+// pools, up to 16 query heads per KV head.  Everything else goes to the
+// vector-ALU kernel.
+//
+// HBM-bound: per sequence 2 * L * Hkv * D * e_kv bytes of K/V are streamed and
+// used exactly once; 4 * G flop per byte (bf16), far below the MFMA roof, so
+// the design goal is bytes in flight, not flops.
+//
+// Work split   one workgroup (4 waves) per (partition, KV head, sequence).
+//              A wave owns whole 32-token tiles (two 16-token blocks) and its
+//              own online-softmax state; no workgroup barrier in the loop.
+// Loads        a (block, KV head) tile is 16 rows * 256 B contiguous (bf16):
+//              each global_load_dwordx4 of a wave reads 1 KB = 4 whole rows,
+//              lane l -> row l/16, 16-byte chunk l%16.  One table lookup per
+//              block, wave-uniform (scalar).
+// K            staged through a wave-private LDS tile (row stride 272 B, so the
+//              16 rows a quarter-wave reads hit distinct banks) and read back
+//              as the A operand of  S^T = K Q^T  (v_mfma_f32_16x16x32_bf16),
+//              the G query heads (padded to 16 columns) sharing every K tile.
+// V            never touches LDS.  Lane (c = l%16, q = l/16) of load i holds
+//              dims 8c..8c+7 of token 4i+q; picking the j-th 16-bit half of
+//              loads 0..7 (v_perm_b32) is exactly the A operand of
+//              O^T[dim 8c+j][head] += V^T P^T  for the token order the QK
+//              product was laid out in (rows of the K tile are permuted on the
+//              LDS read to match), so P goes from accumulator to operand
+//              without leaving its lane.
+// Softmax      log2 domain, running max per head made wave-uniform with two
+//              wave shuffles (lanes l, l^16, l^32, l^48 hold the same head).
+// Split-K      partitions write (max, sum, unnormalised output) to the
+//              workspace; split_reduce_kernel merges them.
 #include "common.h"
+
 namespace aicomp {
-bool decode_mfma_supported(const DecodeArgs&) { return false; }
-int launch_decode_mfma(const DecodeArgs&) { set_error("not built"); return AICOMP_KV_EUNSUPPORTED; }
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int D = 128;
+constexpr int BS = 16;
+constexpr int TILE = 32;               // tokens per wave iteration (two blocks)
+constexpr int NWAVES = 4;
+constexpr int KROW = 272;              // LDS row stride in bytes (256 + 16 pad)
+constexpr int KTILE_BYTES = TILE * KROW;   // 8704 per wave
+constexpr float NEG_BIG = -1.0e30f;
+
+struct MfmaParams {
+    void* out;
+    const void* query;
+    const void* k_pool;
+    const void* v_pool;
+    const int32_t* block_table;
+    int64_t block_table_stride;
+    const int32_t* context_lens;
+    int hq, hkv, group, max_blocks;
+    int64_t num_blocks;
+    float qk_mul;               // scale * log2(e)
+    const float* k_scale;
+    const float* v_scale;
+    int partition_size, num_parts;
+    float* ws_acc;
+    float* ws_ml;
+};
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    bf16x2_t p = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, p);
 }
+
+// 8 fp8 codes -> 8 bf16 (exact: an e4m3 value has 3 mantissa bits)
+__device__ __forceinline__ uint4 fp8x8_to_bf16x8(uint2 r) {
+    uint4 o;
+    auto a = __builtin_amdgcn_cvt_pk_f32_fp8((int)r.x, false);
+    auto b = __builtin_amdgcn_cvt_pk_f32_fp8((int)r.x, true);
+    auto c = __builtin_amdgcn_cvt_pk_f32_fp8((int)r.y, false);
+    auto d = __builtin_amdgcn_cvt_pk_f32_fp8((int)r.y, true);
+    o.x = __builtin_amdgcn_perm(__float_as_uint(a[1]), __float_as_uint(a[0]), 0x07060302u);
+    o.y = __builtin_amdgcn_perm(__float_as_uint(b[1]), __float_as_uint(b[0]), 0x07060302u);
+    o.z = __builtin_amdgcn_perm(__float_as_uint(c[1]), __float_as_uint(c[0]), 0x07060302u);
+    o.w = __builtin_amdgcn_perm(__float_as_uint(d[1]), __float_as_uint(d[0]), 0x07060302u);
+    return o;
+}
+
+template <bool FP8> struct TileRegs;
+template <> struct TileRegs<false> { uint4 r[8]; };
+template <> struct TileRegs<true> { uint2 r[8]; };
+
+// Issue the 8 loads of one 32-token tile of one pool.  blk0/blk1 are the two
+// physical blocks (wave-uniform); lane l reads row l/16, chunk l%16 of each
+// 4-row group.
+template <bool FP8>
+__device__ __forceinline__ void load_tile(TileRegs<FP8>& t, const void* pool, int64_t blk0,
+                                          int64_t blk1, int hkv, int kvh, int lane) {
+    if constexpr (FP8) {
+        const uint2* p0 = (const uint2*)pool + (blk0 * hkv + kvh) * (BS * D / 8) + lane;
+        const uint2* p1 = (const uint2*)pool + (blk1 * hkv + kvh) * (BS * D / 8) + lane;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            t.r[i] = p0[i * 64];
+            t.r[4 + i] = p1[i * 64];
+        }
+    } else {
+        const uint4* p0 = (const uint4*)pool + (blk0 * hkv + kvh) * (BS * D / 8) + lane;
+        const uint4* p1 = (const uint4*)pool + (blk1 * hkv + kvh) * (BS * D / 8) + lane;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            t.r[i] = p0[i * 64];
+            t.r[4 + i] = p1[i * 64];
+        }
+    }
+}
+
+template <bool FP8>
+__device__ __forceinline__ uint4 tile_bf16(const TileRegs<FP8>& t, int i) {
+    if constexpr (FP8) return fp8x8_to_bf16x8(t.r[i]);
+    else return t.r[i];
+}
+
+__device__ __forceinline__ int64_t clamp_block(int b, int64_t num_blocks) {
+    return b < 0 ? 0 : (b >= num_blocks ? num_blocks - 1 : (int64_t)b);
+}
+
+template <bool FP8>
+__global__ void __launch_bounds__(256, 2)
+paged_decode_mfma_kernel(MfmaParams p) {
+    const int part = blockIdx.x;
+    const int kvh = blockIdx.y;
+    const int seq = blockIdx.z;
+    const int tid = threadIdx.x;
+    const int len = min(p.context_lens[seq], p.max_blocks * BS);   // never read past the table row
+    const int start = part * p.partition_size;
+    const int G = p.group;
+
+    if (start >= len) {
+        if (p.num_parts == 1) {   // an unsplit call still owes a defined (zero) output row
+            bf16_t* o = (bf16_t*)p.out + ((int64_t)seq * p.hq + kvh * G) * D;
+            for (int i = tid; i < G * D; i += blockDim.x) o[i].bits = 0;
+        }
+        return;
+    }
+    const int end = min(len, start + p.partition_size);
+    const int ntiles = (end - start + TILE - 1) / TILE;
+
+    const int lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15;      // MFMA row / column index of this lane
+    const int g4 = lane >> 4;       // MFMA k-group of this lane
+
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NWAVES * KTILE_BYTES];
+    __shared__ float sm_m[NWAVES][16];
+    __shared__ float sm_l[NWAVES][16];
+    unsigned char* kt = lds + w * KTILE_BYTES;
+
+    // Q as the B operand of S^T = K Q^T: column = head r16, k-slots = dims 32s + 8*g4 ..
+    bf16x8_t qf[4];
+    {
+        const uint4* qp = (const uint4*)((const bf16_t*)p.query +
+                                         ((int64_t)seq * p.hq + kvh * G + r16) * D + 8 * g4);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (r16 < G) v = qp[s * 4];
+            qf[s] = __builtin_bit_cast(bf16x8_t, v);
+        }
+    }
+    const float cmul = p.qk_mul * (FP8 ? p.k_scale[kvh] : 1.f);
+
+    float m = NEG_BIG, lsum = 0.f;
+    f32x4_t O[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) O[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    const int32_t* table = p.block_table + (int64_t)seq * p.block_table_stride;
+    const int blk_base = start / BS;
+
+    auto tile_blocks = [&](int tt, int64_t& b0, int64_t& b1) {
+        const int i0 = blk_base + 2 * tt;
+        b0 = clamp_block(table[i0], p.num_blocks);
+        b1 = (i0 + 1 < p.max_blocks) ? clamp_block(table[i0 + 1], p.num_blocks) : b0;
+    };
+
+    TileRegs<FP8> kr, vr;
+    if (w < ntiles) {
+        int64_t b0, b1;
+        tile_blocks(w, b0, b1);
+        load_tile<FP8>(kr, p.k_pool, b0, b1, p.hkv, kvh, lane);
+        load_tile<FP8>(vr, p.v_pool, b0, b1, p.hkv, kvh, lane);
+    }
+
+    // LDS addresses: write row = 4i + lane/16, chunk lane%16;
+    // read (sub-tile a, k-step s): row 16a + 4*(r16%4) + r16/4, chunk 4s + g4
+    const int wr_off = (lane >> 4) * KROW + (lane & 15) * 16;
+    const int rd_off = (4 * (r16 & 3) + (r16 >> 2)) * KROW + g4 * 16;
+
+    for (int tt = w; tt < ntiles; tt += NWAVES) {
+        const int tile_start = start + tt * TILE;
+        const bool has_next = tt + NWAVES < ntiles;
+        int64_t nb0 = 0, nb1 = 0;
+        if (has_next) tile_blocks(tt + NWAVES, nb0, nb1);
+
+        // ---- K tile -> LDS, then prefetch the next K tile into the same registers
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            *(uint4*)(kt + wr_off + i * 4 * KROW) = tile_bf16<FP8>(kr, i);
+        if (has_next) load_tile<FP8>(kr, p.k_pool, nb0, nb1, p.hkv, kvh, lane);
+
+        // ---- S^T = K Q^T for the two 16-token sub-tiles
+        f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const uint4 a0 = *(const uint4*)(kt + rd_off + s * 64);
+            const uint4 a1 = *(const uint4*)(kt + rd_off + 16 * KROW + s * 64);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a0), qf[s], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a1), qf[s], s1, 0, 0, 0);
+        }
+        // lane (head r16, g4) now holds tokens tile_start + 16a + 4i + g4 in s_a[i]
+        float sc[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { sc[i] = s0[i] * cmul; sc[4 + i] = s1[i] * cmul; }
+        const bool partial = tile_start + TILE > end;     // wave-uniform
+        if (partial) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int tok = tile_start + 16 * (k >> 2) + 4 * (k & 3) + g4;
+                if (tok >= end) sc[k] = NEG_BIG;
+            }
+        }
+        float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
+                         fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m, mx);
+        const float alpha = exp2f(m - m_new);
+        float pr[8], psum = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            pr[k] = exp2f(sc[k] - m_new);
+            if (partial && sc[k] == NEG_BIG) pr[k] = 0.f;
+            psum += pr[k];
+        }
+        lsum = lsum * alpha + psum;
+        m = m_new;
+        if (__any(alpha != 1.f)) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) O[j] *= alpha;
+        }
+        // P^T as the B operand: k-slot 4a + i <-> token 16a + 4i + g4, this lane's own values
+        uint4 pw;
+        pw.x = pack_bf16(pr[0], pr[1]); pw.y = pack_bf16(pr[2], pr[3]);
+        pw.z = pack_bf16(pr[4], pr[5]); pw.w = pack_bf16(pr[6], pr[7]);
+        const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pw);
+
+        // ---- V: registers -> A operand of O^T += V^T P^T.  Load i of lane (c, q) is token 4i + q.
+        uint4 vv[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            vv[i] = tile_bf16<FP8>(vr, i);
+            if (partial && tile_start + 4 * i + g4 >= end) vv[i] = make_uint4(0, 0, 0, 0);
+        }
+        if (has_next) load_tile<FP8>(vr, p.v_pool, nb0, nb1, p.hkv, kvh, lane);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+            uint4 a;
+            const uint32_t* v0 = (const uint32_t*)&vv[0];
+            a.x = __builtin_amdgcn_perm(v0[4 * 1 + (j >> 1)], v0[4 * 0 + (j >> 1)], sel);
+            a.y = __builtin_amdgcn_perm(v0[4 * 3 + (j >> 1)], v0[4 * 2 + (j >> 1)], sel);
+            a.z = __builtin_amdgcn_perm(v0[4 * 5 + (j >> 1)], v0[4 * 4 + (j >> 1)], sel);
+            a.w = __builtin_amdgcn_perm(v0[4 * 7 + (j >> 1)], v0[4 * 6 + (j >> 1)], sel);
+            O[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), pf, O[j], 0, 0, 0);
+        }
+    }
+
+    // ---- wave result: lane (head r16, g4) holds O^T[dim 32*g4 + 8*i + j][head] in O[j][i]
+    lsum += __shfl_xor(lsum, 16);
+    lsum += __shfl_xor(lsum, 32);
+    float* osm = (float*)kt;        // this wave's own K tile region, G*128 floats <= 8704 bytes
+    if (r16 < G) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float4 a = make_float4(O[0][i], O[1][i], O[2][i], O[3][i]);
+            float4 b = make_float4(O[4][i], O[5][i], O[6][i], O[7][i]);
+            float* dst = osm + r16 * D + 32 * g4 + 8 * i;
+            *(float4*)dst = a;
+            *(float4*)(dst + 4) = b;
+        }
+        if (g4 == 0) { sm_m[w][r16] = m; sm_l[w][r16] = lsum; }
+    }
+    __syncthreads();
+
+    const float vs = FP8 ? p.v_scale[kvh] : 1.f;
+    for (int idx = tid; idx < G * D; idx += 256) {
+        const int h = idx >> 7, dd = idx & 127;
+        float mxw = sm_m[0][h];
+#pragma unroll
+        for (int ww = 1; ww < NWAVES; ++ww) mxw = fmaxf(mxw, sm_m[ww][h]);
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < NWAVES; ++ww) {
+            const float f = exp2f(sm_m[ww][h] - mxw);
+            num = fmaf(f, ((const float*)(lds + ww * KTILE_BYTES))[h * D + dd], num);
+            den = fmaf(f, sm_l[ww][h], den);
+        }
+        const int head = kvh * G + h;
+        if (p.num_parts == 1) {
+            ((bf16_t*)p.out)[((int64_t)seq * p.hq + head) * D + dd].bits =
+                f32_to_bf16(den > 0.f ? vs * num / den : 0.f);
+        } else {
+            const int64_t slot = ((int64_t)seq * p.hq + head) * p.num_parts + part;
+            p.ws_acc[slot * D + dd] = num;
+            if (dd == 0) { p.ws_ml[slot * 2] = mxw; p.ws_ml[slot * 2 + 1] = den; }
+        }
+    }
+}
+
+}  // namespace
+
+bool decode_mfma_supported(const DecodeArgs& a) {
+    const int group = a.hkv > 0 ? a.hq / a.hkv : 0;
+    return a.cu_q_lens == nullptr && a.d == D && a.bs == BS && a.q_dtype == AICOMP_KV_BF16 &&
+           (a.kv_dtype == AICOMP_KV_BF16 || a.kv_dtype == AICOMP_KV_FP8_E4M3) && group >= 1 &&
+           group <= 16 && a.scale > 0.f && a.partition_size % TILE == 0 && a.rows <= 65535 &&
+           a.hkv <= 65535 && ((uintptr_t)a.query % 16 == 0) && ((uintptr_t)a.k_pool % 16 == 0) &&
+           ((uintptr_t)a.v_pool % 16 == 0);
+}
+
+int launch_decode_mfma(const DecodeArgs& a) {
+    MfmaParams p;
+    p.out = a.out; p.query = a.query; p.k_pool = a.k_pool; p.v_pool = a.v_pool;
+    p.block_table = a.block_table; p.block_table_stride = a.block_table_stride;
+    p.context_lens = a.context_lens;
+    p.hq = a.hq; p.hkv = a.hkv; p.group = a.hq / a.hkv; p.max_blocks = a.max_blocks;
+    p.num_blocks = a.num_blocks;
+    p.qk_mul = a.scale * LOG2E;
+    p.k_scale = a.k_scale; p.v_scale = a.v_scale;
+    p.partition_size = a.partition_size; p.num_parts = a.num_parts;
+    p.ws_acc = a.ws.acc; p.ws_ml = a.ws.ml;
+    dim3 grid((unsigned)a.num_parts, (unsigned)a.hkv, (unsigned)a.rows);
+    if (a.kv_dtype == AICOMP_KV_FP8_E4M3)
+        hipLaunchKernelGGL(paged_decode_mfma_kernel<true>, grid, dim3(256), 0, a.stream, p);
+    else
+        hipLaunchKernelGGL(paged_decode_mfma_kernel<false>, grid, dim3(256), 0, a.stream, p);
+    AICOMP_HIP_LAUNCH_CHECK();
+    if (a.num_parts > 1) return launch_split_reduce(a);
+    return AICOMP_KV_OK;
+}
+
+}  // namespace aicomp

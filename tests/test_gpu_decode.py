@@ -115,10 +115,12 @@ def test_decode_invariants(device):
     sh = workloads.Shape("t", 4, 8, 2, 128, ctx_lo=200, ctx_hi=900, kv_std=0.5)
     w = workloads.make_workload("t", device=device, seed=5, shape=sh)
     base = run_decode(w, 256)
-    # split sizes agree to fp32 round-off (outputs are bf16: allow one ulp)
+    # split sizes agree: the merge is exact up to fp32 round-off, what differs is the bf16
+    # rounding of the probabilities (2^-9 relative each, taken against different running
+    # maxima) and of the output; far inside the 1e-2 tolerance
     for ps in (0, 128, 512, 2048):
         o = run_decode(w, ps)
-        assert (o.float() - base.float()).abs().max() <= 2 ** -8 * base.float().abs().max()
+        assert (o.float() - base.float()).abs().max() <= 2e-3
     # moving blocks with the table updated: bit-identical for a fixed partitioning
     nb = w.k_pool.shape[0]
     perm = torch.randperm(nb, device=device)
@@ -191,4 +193,4 @@ def test_config3_long_context_split(device):
     assert_close_attn(got, want, BF16_ATOL, BF16_RTOL, "auto split")
     got1 = to_f64(run_decode(w, w.block_table.shape[1] * 16))      # one partition
     assert_close_attn(got1, want, BF16_ATOL, BF16_RTOL, "unsplit")
-    assert np.abs(got - got1).max() <= 2 ** -7 * np.abs(got1).max()
+    assert np.abs(got - got1).max() <= 2e-3
