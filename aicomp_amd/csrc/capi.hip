@@ -42,10 +42,13 @@ static int check_common(int hq, int hkv, int d, int bs, int max_blocks, int64_t 
 }
 
 static int auto_partition(int64_t rows, int hkv, int bs, int max_blocks) {
+    // Longer partitions amortise a workgroup's start-up and merge; shorter ones give the
+    // 256 CUs enough workgroups when there are few (sequence, KV head) rows.
     const int64_t max_ctx = (int64_t)max_blocks * bs;
-    int ps = 512;
-    // few work items: smaller partitions fill the 256 CUs sooner
-    if (rows * hkv * ((max_ctx + 511) / 512) < 1024) ps = 256;
+    int ps = 256;
+    for (int cand : {1024, 512}) {
+        if (rows * hkv * ((max_ctx + cand - 1) / cand) >= 1024) { ps = cand; break; }
+    }
     ps = (ps + bs - 1) / bs * bs;
     return ps;
 }
@@ -107,7 +110,7 @@ size_t aicomp_paged_decode_workspace_bytes(int batch, int num_q_heads, int num_k
         return 0;
     const int parts = resolve_parts(batch, num_kv_heads, block_size, max_blocks_per_seq, partition_size);
     if (parts <= 1) return 0;
-    return split_workspace_bytes(batch, num_q_heads, head_dim, parts);
+    return split_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, parts);
 }
 
 int aicomp_paged_decode_attn(void* out, const void* query, const void* k_pool, const void* v_pool,
@@ -146,13 +149,13 @@ int aicomp_paged_decode_attn(void* out, const void* query, const void* k_pool, c
     a.num_parts = resolve_parts(batch, num_kv_heads, block_size, max_blocks_per_seq, a.partition_size);
     a.stream = (hipStream_t)stream;
     if (a.num_parts > 1) {
-        const size_t need = split_workspace_bytes(a.rows, a.hq, a.d, a.num_parts);
+        const size_t need = split_workspace_bytes(a.rows, a.hq, a.hkv, a.d, a.num_parts);
         AICOMP_REQUIRE(workspace && workspace_bytes >= need, AICOMP_KV_EWORKSPACE,
                        "paged_decode_attn: workspace of %zu bytes needed, %zu given", need,
                        workspace ? workspace_bytes : (size_t)0);
         AICOMP_REQUIRE((uintptr_t)workspace % 16 == 0, AICOMP_KV_EINVAL,
                        "paged_decode_attn: workspace must be 16-byte aligned");
-        a.ws = split_workspace_view(workspace, a.rows, a.hq, a.d, a.num_parts);
+        a.ws = split_workspace_view(workspace, a.rows, a.hq, a.hkv, a.d, a.num_parts);
     }
     if (decode_mfma_supported(a)) return launch_decode_mfma(a);
     return launch_decode_generic(a);

@@ -241,9 +241,11 @@ paged_attn_generic_kernel(GenericParams p) {
 }
 
 // Split-K merge: out = sum_p 2^(m_p - M) acc_p / sum_p 2^(m_p - M) l_p, M = max_p m_p.
-// One workgroup per (row, head); only the partitions that hold tokens are read.
+// One workgroup per (row, head); only the partitions that hold tokens are read.  The
+// weights 2^(m_p - M) / sum are computed once (one lane per partition, wave reduction) and
+// parked in LDS; the accumulation loop then issues independent loads.
 template <typename Q_T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(128)
 split_reduce_kernel(Q_T* __restrict__ out, const float* __restrict__ ws_acc,
                     const float* __restrict__ ws_ml, const int32_t* __restrict__ context_lens,
                     const int32_t* __restrict__ cu_q_lens, int num_seqs, int hq, int group, int d,
@@ -254,24 +256,52 @@ split_reduce_kernel(Q_T* __restrict__ out, const float* __restrict__ ws_acc,
     row_info(row, cu_q_lens, context_lens, num_seqs, seq, len);
     const int np = min(num_parts, (len + partition_size - 1) / partition_size);
     const int64_t slot0 = (row * hq + head) * num_parts;
+    __shared__ float wgt[1024];
+    __shared__ float red[2][2];
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    // pass 1: max over partitions
     float mx = NEG_BIG;
-    for (int pi = 0; pi < np; ++pi) mx = fmaxf(mx, ws_ml[(slot0 + pi) * 2]);
+    for (int pi = tid; pi < np; pi += blockDim.x) mx = fmaxf(mx, ws_ml[(slot0 + pi) * 2]);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    if (lane == 0) red[0][wv] = mx;
+    __syncthreads();
+    mx = fmaxf(red[0][0], red[0][1]);
+    // pass 2: weights and their sum (np <= 1024 partitions are cached in LDS)
     float den = 0.f;
-    for (int pi = 0; pi < np; ++pi)
-        den = fmaf(exp2f(ws_ml[(slot0 + pi) * 2] - mx), ws_ml[(slot0 + pi) * 2 + 1], den);
+    for (int pi = tid; pi < np; pi += blockDim.x) {
+        const float f = exp2f(ws_ml[(slot0 + pi) * 2] - mx);
+        if (pi < 1024) wgt[pi] = f;
+        den = fmaf(f, ws_ml[(slot0 + pi) * 2 + 1], den);
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) den += __shfl_xor(den, o);
+    if (lane == 0) red[1][wv] = den;
+    __syncthreads();
+    den = red[1][0] + red[1][1];
     const float vs = v_scale ? v_scale[head / group] : 1.f;
     const float inv = den > 0.f ? vs / den : 0.f;
-    for (int dd = threadIdx.x; dd < d; dd += blockDim.x) {
+    for (int dd = tid; dd < d; dd += blockDim.x) {
         float num = 0.f;
-        for (int pi = 0; pi < np; ++pi)
-            num = fmaf(exp2f(ws_ml[(slot0 + pi) * 2] - mx), ws_acc[(slot0 + pi) * d + dd], num);
+        const float* a = ws_acc + slot0 * d + dd;
+        int pi = 0;
+        for (; pi + 4 <= np && pi + 4 <= 1024; pi += 4) {
+            const float a0 = a[(int64_t)pi * d], a1 = a[(int64_t)(pi + 1) * d];
+            const float a2 = a[(int64_t)(pi + 2) * d], a3 = a[(int64_t)(pi + 3) * d];
+            num = fmaf(wgt[pi], a0, num); num = fmaf(wgt[pi + 1], a1, num);
+            num = fmaf(wgt[pi + 2], a2, num); num = fmaf(wgt[pi + 3], a3, num);
+        }
+        for (; pi < np; ++pi) {
+            const float f = pi < 1024 ? wgt[pi] : exp2f(ws_ml[(slot0 + pi) * 2] - mx);
+            num = fmaf(f, a[(int64_t)pi * d], num);
+        }
         store_elem<Q_T>(out + (row * hq + head) * d + dd, num * inv);
     }
 }
 
 int launch_split_reduce(const DecodeArgs& a) {
     dim3 grid((unsigned)a.rows, (unsigned)a.hq);
-    const int threads = a.d <= 64 ? 64 : (a.d <= 128 ? 128 : 256);
+    const int threads = 128;
     const int group = a.hq / a.hkv;
     if (a.q_dtype == AICOMP_KV_F32)
         hipLaunchKernelGGL(split_reduce_kernel<float>, grid, dim3(threads), 0, a.stream,

@@ -34,7 +34,9 @@
 // Softmax      log2 domain, running max per head made wave-uniform with two
 //              wave shuffles (lanes l, l^16, l^32, l^48 hold the same head).
 // Split-K      partitions write (max, sum, unnormalised output) to the
-//              workspace; split_reduce_kernel merges them.
+//              workspace; the workgroup that finishes a (sequence, KV head)'s
+//              last partition (device-scope counter) merges them in the same
+//              launch, so a decode call is one kernel.
 #include "common.h"
 
 namespace aicomp {
@@ -67,6 +69,7 @@ struct MfmaParams {
     const float* k_scale;
     const float* v_scale;
     int partition_size, num_parts;
+    int* ws_counters;
     float* ws_acc;
     float* ws_ml;
 };
@@ -129,19 +132,152 @@ __device__ __forceinline__ int64_t clamp_block(int b, int64_t num_blocks) {
     return b < 0 ? 0 : (b >= num_blocks ? num_blocks - 1 : (int64_t)b);
 }
 
+// Per-wave running state of the online softmax and the output accumulators.
+struct WaveState {
+    float m, lsum;
+    f32x4_t O[8];
+};
+
+// One 32-token tile: K registers -> LDS -> S^T = K Q^T -> online softmax -> O^T += V^T P^T.
+// NEXT: prefetch the wave's next tile (blocks nb0/nb1) into the same registers.
+// MASK: the tile crosses `end`; scores beyond it are dropped and their V rows zeroed.
+template <bool FP8, bool NEXT, bool MASK>
+__device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, TileRegs<FP8>& vr,
+                                             const bf16x8_t (&qf)[4], unsigned char* kt, int wr_off,
+                                             int rd_off, const void* k_pool, const void* v_pool,
+                                             int64_t nb0, int64_t nb1, int hkv, int kvh, int lane,
+                                             int g4, int tile_start, int end, float cmul) {
+#ifdef EXP_LOADS_ONLY
+    {
+        uint4 x = make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { uint4 a = tile_bf16<FP8>(kr, i); x.x ^= a.x; x.y ^= a.y; x.z ^= a.z; x.w ^= a.w; }
+        if (NEXT) load_tile<FP8>(kr, k_pool, nb0, nb1, hkv, kvh, lane);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { uint4 a = tile_bf16<FP8>(vr, i); x.x ^= a.x; x.y ^= a.y; x.z ^= a.z; x.w ^= a.w; }
+        if (NEXT) load_tile<FP8>(vr, v_pool, nb0, nb1, hkv, kvh, lane);
+        st.O[0][0] += __uint_as_float(x.x ^ x.y ^ x.z ^ x.w);
+        return;
+    }
+#endif
+    // ---- K tile -> LDS, then prefetch the next K tile into the same registers
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        *(uint4*)(kt + wr_off + i * 4 * KROW) = tile_bf16<FP8>(kr, i);
+    if (NEXT) load_tile<FP8>(kr, k_pool, nb0, nb1, hkv, kvh, lane);
+
+    // ---- S^T = K Q^T for the two 16-token sub-tiles
+    f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        const uint4 a0 = *(const uint4*)(kt + rd_off + s * 64);
+        const uint4 a1 = *(const uint4*)(kt + rd_off + 16 * KROW + s * 64);
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a0), qf[s], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a1), qf[s], s1, 0, 0, 0);
+    }
+    // lane (head r16, g4) now holds tokens tile_start + 16a + 4i + g4 in s_a[i]
+    float sc[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { sc[i] = s0[i] * cmul; sc[4 + i] = s1[i] * cmul; }
+    if (MASK) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int tok = tile_start + 16 * (k >> 2) + 4 * (k & 3) + g4;
+            if (tok >= end) sc[k] = NEG_BIG;
+        }
+    }
+    float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
+                     fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(st.m, mx);
+    const float alpha = exp2f(st.m - m_new);
+    float pr[8], psum = 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        pr[k] = exp2f(sc[k] - m_new);
+        if (MASK && sc[k] == NEG_BIG) pr[k] = 0.f;
+        psum += pr[k];
+    }
+    st.lsum = st.lsum * alpha + psum;
+    st.m = m_new;
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) st.O[j] *= alpha;
+    }
+    // P^T as the B operand: k-slot 4a + i <-> token 16a + 4i + g4, this lane's own values
+    uint4 pw;
+    pw.x = pack_bf16(pr[0], pr[1]); pw.y = pack_bf16(pr[2], pr[3]);
+    pw.z = pack_bf16(pr[4], pr[5]); pw.w = pack_bf16(pr[6], pr[7]);
+    const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pw);
+
+    // ---- V: registers -> A operand of O^T += V^T P^T.  Load i of lane (c, q) is token 4i + q.
+    uint4 vv[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        vv[i] = tile_bf16<FP8>(vr, i);
+        if (MASK && tile_start + 4 * i + g4 >= end) vv[i] = make_uint4(0, 0, 0, 0);
+    }
+    uint4 af[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+        const uint32_t* v0 = (const uint32_t*)&vv[0];
+        af[j].x = __builtin_amdgcn_perm(v0[4 * 1 + (j >> 1)], v0[4 * 0 + (j >> 1)], sel);
+        af[j].y = __builtin_amdgcn_perm(v0[4 * 3 + (j >> 1)], v0[4 * 2 + (j >> 1)], sel);
+        af[j].z = __builtin_amdgcn_perm(v0[4 * 5 + (j >> 1)], v0[4 * 4 + (j >> 1)], sel);
+        af[j].w = __builtin_amdgcn_perm(v0[4 * 7 + (j >> 1)], v0[4 * 6 + (j >> 1)], sel);
+    }
+    if (NEXT) load_tile<FP8>(vr, v_pool, nb0, nb1, hkv, kvh, lane);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+        st.O[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, af[j]), pf, st.O[j], 0, 0, 0);
+}
+
 template <bool FP8>
-__global__ void __launch_bounds__(256, 2)
+#ifndef EXP_WPS
+#define EXP_WPS 2
+#endif
+__global__ void __launch_bounds__(256, EXP_WPS)
 paged_decode_mfma_kernel(MfmaParams p) {
-    const int part = blockIdx.x;
-    const int kvh = blockIdx.y;
+    // KV head fastest: the workgroups launched together read the Hkv slices of the same
+    // physical blocks, i.e. one contiguous Hkv*4 KB piece of each pool
+    const int kvh = blockIdx.x;
+    const int part = blockIdx.y;
     const int seq = blockIdx.z;
     const int tid = threadIdx.x;
-    const int len = min(p.context_lens[seq], p.max_blocks * BS);   // never read past the table row
-    const int start = part * p.partition_size;
+    const int lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15;      // MFMA row / column index of this lane
+    const int g4 = lane >> 4;       // MFMA k-group of this lane
     const int G = p.group;
+    const int start = part * p.partition_size;
+    const int blk_base = start / BS;
 
+    // Prologue loads, all issued before anything waits: the context length (scalar), the
+    // partition's slice of the block table (one coalesced vector load: lane i holds entry
+    // blk_base + i, later picked out with v_readlane, so the loop has no table loads at
+    // all) and the query rows.
+    const int32_t* table = p.block_table + (int64_t)seq * p.block_table_stride;
+    int tab_first = 0;                       // first entry (relative to blk_base) held in `tab`
+    int tab = (blk_base + lane < p.max_blocks) ? table[blk_base + lane] : 0;
+
+    // Q as the B operand of S^T = K Q^T: column = head r16, k-slots = dims 32s + 8*g4 ..
+    bf16x8_t qf[4];
+    {
+        const uint4* qp = (const uint4*)((const bf16_t*)p.query +
+                                         ((int64_t)seq * p.hq + kvh * G + min(r16, G - 1)) * D + 8 * g4);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            uint4 v = qp[s * 4];
+            if (r16 >= G) v = make_uint4(0, 0, 0, 0);
+            qf[s] = __builtin_bit_cast(bf16x8_t, v);
+        }
+    }
+
+    const int len = min(p.context_lens[seq], p.max_blocks * BS);   // never read past the table row
     if (start >= len) {
-        if (p.num_parts == 1) {   // an unsplit call still owes a defined (zero) output row
+        if (len <= 0 && part == 0) {   // nothing to attend to: the output row is defined as zero
             bf16_t* o = (bf16_t*)p.out + ((int64_t)seq * p.hq + kvh * G) * D;
             for (int i = tid; i < G * D; i += blockDim.x) o[i].bits = 0;
         }
@@ -150,135 +286,65 @@ paged_decode_mfma_kernel(MfmaParams p) {
     const int end = min(len, start + p.partition_size);
     const int ntiles = (end - start + TILE - 1) / TILE;
 
-    const int lane = tid & 63;
-    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int r16 = lane & 15;      // MFMA row / column index of this lane
-    const int g4 = lane >> 4;       // MFMA k-group of this lane
-
     __shared__ __attribute__((aligned(16))) unsigned char lds[NWAVES * KTILE_BYTES];
     __shared__ float sm_m[NWAVES][16];
     __shared__ float sm_l[NWAVES][16];
     unsigned char* kt = lds + w * KTILE_BYTES;
 
-    // Q as the B operand of S^T = K Q^T: column = head r16, k-slots = dims 32s + 8*g4 ..
-    bf16x8_t qf[4];
-    {
-        const uint4* qp = (const uint4*)((const bf16_t*)p.query +
-                                         ((int64_t)seq * p.hq + kvh * G + r16) * D + 8 * g4);
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (r16 < G) v = qp[s * 4];
-            qf[s] = __builtin_bit_cast(bf16x8_t, v);
-        }
-    }
     const float cmul = p.qk_mul * (FP8 ? p.k_scale[kvh] : 1.f);
 
-    float m = NEG_BIG, lsum = 0.f;
-    f32x4_t O[8];
+    WaveState st;
+    st.m = NEG_BIG; st.lsum = 0.f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) O[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < 8; ++j) st.O[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    const int32_t* table = p.block_table + (int64_t)seq * p.block_table_stride;
-    const int blk_base = start / BS;
-
+    // physical blocks of tile tt (wave-uniform); the held table slice is refilled every 64 blocks
     auto tile_blocks = [&](int tt, int64_t& b0, int64_t& b1) {
-        const int i0 = blk_base + 2 * tt;
-        b0 = clamp_block(table[i0], p.num_blocks);
-        b1 = (i0 + 1 < p.max_blocks) ? clamp_block(table[i0 + 1], p.num_blocks) : b0;
+        const int i0 = 2 * tt;
+        if (i0 - tab_first >= 64) {
+            tab_first = i0;
+            tab = (blk_base + i0 + lane < p.max_blocks) ? table[blk_base + i0 + lane] : 0;
+            __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0) here, so the common path never waits on `tab`
+        }
+        b0 = clamp_block(__builtin_amdgcn_readlane(tab, i0 - tab_first), p.num_blocks);
+        b1 = clamp_block(__builtin_amdgcn_readlane(tab, i0 + 1 - tab_first), p.num_blocks);
     };
-
-    TileRegs<FP8> kr, vr;
-    if (w < ntiles) {
-        int64_t b0, b1;
-        tile_blocks(w, b0, b1);
-        load_tile<FP8>(kr, p.k_pool, b0, b1, p.hkv, kvh, lane);
-        load_tile<FP8>(vr, p.v_pool, b0, b1, p.hkv, kvh, lane);
-    }
 
     // LDS addresses: write row = 4i + lane/16, chunk lane%16;
     // read (sub-tile a, k-step s): row 16a + 4*(r16%4) + r16/4, chunk 4s + g4
     const int wr_off = (lane >> 4) * KROW + (lane & 15) * 16;
     const int rd_off = (4 * (r16 & 3) + (r16 >> 2)) * KROW + g4 * 16;
 
-    for (int tt = w; tt < ntiles; tt += NWAVES) {
+    if (w < ntiles) {
+        TileRegs<FP8> kr, vr;
+        int64_t b0, b1;
+        tile_blocks(w, b0, b1);
+        // Q must have landed before the tile loads are issued: the loop's waits then count
+        // only tile loads, so a wave computes on tile t while tile t+1 is still in flight.
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+        load_tile<FP8>(kr, p.k_pool, b0, b1, p.hkv, kvh, lane);
+        load_tile<FP8>(vr, p.v_pool, b0, b1, p.hkv, kvh, lane);
+        int tt = w;
+        for (; tt + NWAVES < ntiles; tt += NWAVES) {      // steady state: never the partition's last tile
+            tile_blocks(tt + NWAVES, b0, b1);
+            process_tile<FP8, true, false>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, b0,
+                                           b1, p.hkv, kvh, lane, g4, start + tt * TILE, end, cmul);
+        }
         const int tile_start = start + tt * TILE;
-        const bool has_next = tt + NWAVES < ntiles;
-        int64_t nb0 = 0, nb1 = 0;
-        if (has_next) tile_blocks(tt + NWAVES, nb0, nb1);
-
-        // ---- K tile -> LDS, then prefetch the next K tile into the same registers
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-            *(uint4*)(kt + wr_off + i * 4 * KROW) = tile_bf16<FP8>(kr, i);
-        if (has_next) load_tile<FP8>(kr, p.k_pool, nb0, nb1, p.hkv, kvh, lane);
-
-        // ---- S^T = K Q^T for the two 16-token sub-tiles
-        f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const uint4 a0 = *(const uint4*)(kt + rd_off + s * 64);
-            const uint4 a1 = *(const uint4*)(kt + rd_off + 16 * KROW + s * 64);
-            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a0), qf[s], s0, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a1), qf[s], s1, 0, 0, 0);
-        }
-        // lane (head r16, g4) now holds tokens tile_start + 16a + 4i + g4 in s_a[i]
-        float sc[8];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) { sc[i] = s0[i] * cmul; sc[4 + i] = s1[i] * cmul; }
-        const bool partial = tile_start + TILE > end;     // wave-uniform
-        if (partial) {
-#pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const int tok = tile_start + 16 * (k >> 2) + 4 * (k & 3) + g4;
-                if (tok >= end) sc[k] = NEG_BIG;
-            }
-        }
-        float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
-                         fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-        mx = fmaxf(mx, __shfl_xor(mx, 16));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m, mx);
-        const float alpha = exp2f(m - m_new);
-        float pr[8], psum = 0.f;
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            pr[k] = exp2f(sc[k] - m_new);
-            if (partial && sc[k] == NEG_BIG) pr[k] = 0.f;
-            psum += pr[k];
-        }
-        lsum = lsum * alpha + psum;
-        m = m_new;
-        if (__any(alpha != 1.f)) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) O[j] *= alpha;
-        }
-        // P^T as the B operand: k-slot 4a + i <-> token 16a + 4i + g4, this lane's own values
-        uint4 pw;
-        pw.x = pack_bf16(pr[0], pr[1]); pw.y = pack_bf16(pr[2], pr[3]);
-        pw.z = pack_bf16(pr[4], pr[5]); pw.w = pack_bf16(pr[6], pr[7]);
-        const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pw);
-
-        // ---- V: registers -> A operand of O^T += V^T P^T.  Load i of lane (c, q) is token 4i + q.
-        uint4 vv[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            vv[i] = tile_bf16<FP8>(vr, i);
-            if (partial && tile_start + 4 * i + g4 >= end) vv[i] = make_uint4(0, 0, 0, 0);
-        }
-        if (has_next) load_tile<FP8>(vr, p.v_pool, nb0, nb1, p.hkv, kvh, lane);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
-            uint4 a;
-            const uint32_t* v0 = (const uint32_t*)&vv[0];
-            a.x = __builtin_amdgcn_perm(v0[4 * 1 + (j >> 1)], v0[4 * 0 + (j >> 1)], sel);
-            a.y = __builtin_amdgcn_perm(v0[4 * 3 + (j >> 1)], v0[4 * 2 + (j >> 1)], sel);
-            a.z = __builtin_amdgcn_perm(v0[4 * 5 + (j >> 1)], v0[4 * 4 + (j >> 1)], sel);
-            a.w = __builtin_amdgcn_perm(v0[4 * 7 + (j >> 1)], v0[4 * 6 + (j >> 1)], sel);
-            O[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), pf, O[j], 0, 0, 0);
-        }
+        if (tile_start + TILE > end)
+            process_tile<FP8, false, true>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
+                                           p.hkv, kvh, lane, g4, tile_start, end, cmul);
+        else
+            process_tile<FP8, false, false>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
+                                            p.hkv, kvh, lane, g4, tile_start, end, cmul);
     }
+    const float m = st.m;
+    float lsum = st.lsum;
+    f32x4_t (&O)[8] = st.O;
+#ifdef EXP_NO_EPI
+    if (p.num_parts == 12345) ((float*)p.out)[tid] = m + lsum + O[0][0] + O[1][1] + O[2][2] + O[3][3] + O[4][0] + O[5][1] + O[6][2] + O[7][3];
+    return;
+#endif
 
     // ---- wave result: lane (head r16, g4) holds O^T[dim 32*g4 + 8*i + j][head] in O[j][i]
     lsum += __shfl_xor(lsum, 16);
@@ -298,6 +364,8 @@ paged_decode_mfma_kernel(MfmaParams p) {
     __syncthreads();
 
     const float vs = FP8 ? p.v_scale[kvh] : 1.f;
+    const int nvalid = (len + p.partition_size - 1) / p.partition_size;   // partitions holding tokens
+    const bool direct = p.num_parts == 1;     // unsplit call: no merge needed
     for (int idx = tid; idx < G * D; idx += 256) {
         const int h = idx >> 7, dd = idx & 127;
         float mxw = sm_m[0][h];
@@ -311,7 +379,7 @@ paged_decode_mfma_kernel(MfmaParams p) {
             den = fmaf(f, sm_l[ww][h], den);
         }
         const int head = kvh * G + h;
-        if (p.num_parts == 1) {
+        if (direct) {
             ((bf16_t*)p.out)[((int64_t)seq * p.hq + head) * D + dd].bits =
                 f32_to_bf16(den > 0.f ? vs * num / den : 0.f);
         } else {
@@ -329,7 +397,7 @@ bool decode_mfma_supported(const DecodeArgs& a) {
     return a.cu_q_lens == nullptr && a.d == D && a.bs == BS && a.q_dtype == AICOMP_KV_BF16 &&
            (a.kv_dtype == AICOMP_KV_BF16 || a.kv_dtype == AICOMP_KV_FP8_E4M3) && group >= 1 &&
            group <= 16 && a.scale > 0.f && a.partition_size % TILE == 0 && a.rows <= 65535 &&
-           a.hkv <= 65535 && ((uintptr_t)a.query % 16 == 0) && ((uintptr_t)a.k_pool % 16 == 0) &&
+           a.num_parts <= 65535 && ((uintptr_t)a.query % 16 == 0) && ((uintptr_t)a.k_pool % 16 == 0) &&
            ((uintptr_t)a.v_pool % 16 == 0);
 }
 
@@ -343,8 +411,8 @@ int launch_decode_mfma(const DecodeArgs& a) {
     p.qk_mul = a.scale * LOG2E;
     p.k_scale = a.k_scale; p.v_scale = a.v_scale;
     p.partition_size = a.partition_size; p.num_parts = a.num_parts;
-    p.ws_acc = a.ws.acc; p.ws_ml = a.ws.ml;
-    dim3 grid((unsigned)a.num_parts, (unsigned)a.hkv, (unsigned)a.rows);
+    p.ws_counters = a.ws.counters; p.ws_acc = a.ws.acc; p.ws_ml = a.ws.ml;
+    dim3 grid((unsigned)a.hkv, (unsigned)a.num_parts, (unsigned)a.rows);
     if (a.kv_dtype == AICOMP_KV_FP8_E4M3)
         hipLaunchKernelGGL(paged_decode_mfma_kernel<true>, grid, dim3(256), 0, a.stream, p);
     else

@@ -1,0 +1,262 @@
+"""Benchmark of the paged KV-cache attention path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+
+A step is one pass of the hot path over one synthetic batch of the Llama-3-8B
+decode shape (batch 64, 32 query / 8 KV heads, head_dim 128, block 16, context
+uniform in [512,4096], bf16): KV append of one token per sequence, then paged
+decode attention.  All inputs are resident in HBM before the timed region.
+Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+METRIC = "decode-attn HBM GB/s (% peak) + tokens/s, Llama-3-8B paged KV, 1 GPU"
+
+# HBM bytes per decode launch of the Llama-3-8B shape from rocprofv3 --pmc
+# (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); None until measured.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def _events(n):
+    import torch
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def run_decode_config(name, steps, warmup, dev):
+    """Append + decode for one workload; returns timing and algorithmic figures."""
+    import torch
+    from aicomp_amd import ops, workloads
+    w = workloads.make_workload(name, device=dev)
+    npre = w.num_prefill_seqs
+    S = w.num_seqs
+    # decode part: the sequences that add one token
+    qd = w.query[int(w.cu_q_lens[npre]):].contiguous()
+    btd = w.block_table[npre:].contiguous()
+    cld = w.context_lens[npre:].contiguous()
+    outd = torch.empty_like(qd)
+    if npre:
+        T_pre = int(w.cu_q_lens[npre])
+        qp = w.query[:T_pre].contiguous()
+        outp = torch.empty_like(qp)
+        btp = w.block_table[:npre].contiguous()
+        clp = w.context_lens[:npre].contiguous()
+        cup = w.cu_q_lens[:npre + 1].contiguous()
+        max_q = max(w.new_list[:npre])
+
+    def step(ev=None):
+        if ev: ev[0].record()
+        ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping, w.k_scale, w.v_scale)
+        if ev: ev[1].record()
+        if npre:
+            ops.paged_prefill_attn(outp, qp, w.k_pool, w.v_pool, btp, clp, cup, w.scale, max_q_len=max_q)
+        if ev: ev[2].record()
+        ops.paged_decode_attn(outd, qd, w.k_pool, w.v_pool, btd, cld, w.scale, w.k_scale, w.v_scale)
+        if ev: ev[3].record()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    evs = [_events(4) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(evs[i])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    t_app = statistics.mean(e[0].elapsed_time(e[1]) for e in evs) * 1e-3
+    t_pre = statistics.mean(e[1].elapsed_time(e[2]) for e in evs) * 1e-3
+    t_dec = statistics.mean(e[2].elapsed_time(e[3]) for e in evs) * 1e-3
+    res = {
+        "workload": name, "ms_per_step": wall / steps * 1e3,
+        "append_us": t_app * 1e6, "append_bytes": w.append_bytes(),
+        "append_GBs": w.append_bytes() / t_app / 1e9,
+        "decode_us": t_dec * 1e6, "decode_bytes": w.decode_kv_bytes(),
+        "decode_GBs": w.decode_kv_bytes() / t_dec / 1e9,
+        "decode_frac_hbm_peak": w.decode_kv_bytes() / t_dec / 1e9 / HBM_PEAK_GBS,
+        "decode_tokens_per_s": (S - npre) / t_dec,
+        "partition_size": ops.decode_partition_size(S - npre, w.shape.num_q_heads, w.shape.num_kv_heads,
+                                                    w.shape.head_dim, w.shape.block_size, btd.shape[1],
+                                                    qd.dtype, w.k_pool.dtype),
+        "kv_dtype": str(w.k_pool.dtype).replace("torch.", ""),
+    }
+    if npre:
+        res.update({"prefill_us": t_pre * 1e6, "prefill_flops": w.prefill_flops(),
+                    "prefill_TFLOPs": w.prefill_flops() / t_pre / 1e12,
+                    "prefill_frac_mfma_peak": w.prefill_flops() / t_pre / 1e12 / MFMA_BF16_PEAK_TFLOPS})
+    return res, w
+
+
+def profile_target(which, steps, warmup, dev):
+    """Launch one kernel of the path repeatedly, for rocprofv3 (--kernel-trace / --pmc).
+    "copy" is a plain device copy of exactly 1 GiB: the counter calibration."""
+    import torch
+    from aicomp_amd import ops, workloads
+    if which == "copy":
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(warmup + steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(f"copy: {steps + warmup} launches of {src.numel()} bytes read + {dst.numel()} bytes written")
+        return
+    name = {"decode": "llama3_8b_decode", "append": "chunked_prefill_mixed", "prefill": "chunked_prefill_mixed",
+            "decode_fp8": "llama3_70b_decode_fp8", "decode_long": "long_context_skewed"}[which]
+    w = workloads.make_workload(name, device=dev)
+    ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping, w.k_scale, w.v_scale)
+    npre = w.num_prefill_seqs
+    t0 = int(w.cu_q_lens[npre])
+    if which.startswith("decode"):
+        q = w.query[t0:].contiguous()
+        out = torch.empty_like(q)
+        bt, cl = w.block_table[npre:].contiguous(), w.context_lens[npre:].contiguous()
+        fn = lambda: ops.paged_decode_attn(out, q, w.k_pool, w.v_pool, bt, cl, w.scale, w.k_scale, w.v_scale)
+        info = f"{w.decode_kv_bytes()} algorithmic bytes per launch"
+    elif which == "append":
+        fn = lambda: ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping)
+        info = f"{w.append_bytes()} algorithmic bytes per launch"
+    else:
+        q = w.query[:t0].contiguous()
+        out = torch.empty_like(q)
+        bt, cl, cu = w.block_table[:npre].contiguous(), w.context_lens[:npre].contiguous(), w.cu_q_lens[:npre + 1].contiguous()
+        mq = max(w.new_list[:npre])
+        fn = lambda: ops.paged_prefill_attn(out, q, w.k_pool, w.v_pool, bt, cl, cu, w.scale, max_q_len=mq)
+        info = f"{w.prefill_flops()} algorithmic flop per launch"
+    for _ in range(warmup + steps):
+        fn()
+    torch.cuda.synchronize()
+    print(f"{which} ({name}): {steps + warmup} launches, {info}")
+
+
+def cpu_baseline(w, budget_s=20.0):
+    """The reference's CPU path (gather -> repeat_kv -> contiguous -> SDPA), restated in
+    oracle/contiguous_ref.py, timed on the host cores over a bounded sample of the batch."""
+    import torch
+    from oracle import contiguous_ref as cref
+    threads = torch.get_num_threads()
+    npre = w.num_prefill_seqs
+    q = w.query[int(w.cu_q_lens[npre]):].cpu()
+    bt = w.block_table[npre:].cpu()
+    cl = w.context_lens[npre:].cpu()
+    kp, vp = w.k_pool.cpu(), w.v_pool.cpu()
+    ks = None if w.k_scale is None else w.k_scale.cpu()
+    vs = None if w.v_scale is None else w.v_scale.cpu()
+    B = q.shape[0]
+    n = min(B, 8)
+
+    def run(nseq):
+        t0 = time.perf_counter()
+        cref.reference_cpu_decode(q[:nseq], kp, vp, bt[:nseq], cl[:nseq], w.scale, ks, vs,
+                                  compute_dtype=q.dtype)
+        return time.perf_counter() - t0
+
+    t1 = run(n)
+    # sample: as many sequences as fit ~budget with 3 warmups + >= 3 timed repetitions
+    per_seq = t1 / n
+    nseq = int(max(1, min(B, budget_s / (6 * per_seq))))
+    reps = int(max(3, min(10, budget_s / (per_seq * nseq) - 3)))
+    for _ in range(2):
+        run(nseq)
+    ts = sorted(run(nseq) for _ in range(reps))
+    med = ts[len(ts) // 2]
+    e = w.k_pool.element_size()
+    s = w.shape
+    byts = sum(2 * L * s.num_kv_heads * s.head_dim * e for L in w.ctx_list[npre:npre + nseq])
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"value": byts / med / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "tokens_per_s": nseq / med,
+            "sample": f"first {nseq} of {B} sequences of the same batch, decode attention only "
+                      f"(gather blocks -> repeat_kv -> contiguous -> torch SDPA, {str(q.dtype).replace('torch.', '')}), "
+                      f"2 warmups, median of {reps}; {med * 1e3:.1f} ms per pass; "
+                      f"cpu '{model}', os.cpu_count()={os.cpu_count()}, torch threads={threads}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
+    ap.add_argument("--only", choices=["decode", "append", "copy", "prefill", "decode_fp8", "decode_long"],
+                    help="profiling target: launch just this kernel --steps times (no JSON line)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU only (asked for --gpus {args.gpus}); "
+              "the path shards by sequence or by KV head with no communication, but no "
+              "multi-GPU code is part of it.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from aicomp_amd import _lib
+    _lib.load()     # fails loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+
+    if args.only:
+        profile_target(args.only, args.steps, args.warmup, dev)
+        return
+    main_res, w = run_decode_config("llama3_8b_decode", args.steps, args.warmup, dev)
+    s = w.shape
+    line = {
+        "metric": METRIC,
+        "value": main_res["decode_bytes"] / (main_res["ms_per_step"] * 1e-3) / 1e9,
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": main_res["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "llama3_8b_decode: batch 64, 32 query / 8 KV heads, head_dim 128, "
+                               "block 16, context uniform [512,4096] seed 0, bf16; step = KV append "
+                               "of 64 rows + paged decode attention",
+                   "batch": s.batch, "partition_size": main_res["partition_size"],
+                   "kv_bytes_per_step": main_res["decode_bytes"]},
+        "tokens_per_s": s.batch / (main_res["ms_per_step"] * 1e-3),
+        "pct_hbm_peak": 100.0 * main_res["decode_bytes"] / (main_res["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "roofline": {"kernel": "paged_decode_mfma_kernel<bf16> + split_reduce_kernel (one decode call)",
+                     "bound": "hbm", "achieved": main_res["decode_GBs"], "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": main_res["decode_GBs"] / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES,
+                     "algorithmic_bytes": main_res["decode_bytes"],
+                     "avg_launch_us": main_res["decode_us"]},
+        "append": {"us": main_res["append_us"], "GB/s": main_res["append_GBs"],
+                   "bytes": main_res["append_bytes"]},
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(w)
+    del w
+    torch.cuda.empty_cache()
+    if not args.no_extra:
+        extra = []
+        for name in ("decode_fp32_small", "long_context_skewed", "chunked_prefill_mixed",
+                     "llama3_70b_decode_fp8"):
+            r, ww = run_decode_config(name, max(10, args.steps // 4), max(3, args.warmup // 4), dev)
+            del ww
+            torch.cuda.empty_cache()
+            extra.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})
+        line["other_workloads"] = extra
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

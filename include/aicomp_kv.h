@@ -91,7 +91,13 @@ int aicomp_kv_append(const void* key, const void* value,
  *                   partial (max, sum, output) triples.
  *   workspace       device scratch of at least
  *                   aicomp_paged_decode_workspace_bytes(...) bytes (may be NULL
- *                   when that returns 0)
+ *                   when that returns 0), 16-byte aligned.  Its leading
+ *                   batch * num_kv_heads int32 words are completion counters:
+ *                   they must be ZERO before the first call that uses the
+ *                   buffer and every call leaves them zero again, so one
+ *                   zero-filled allocation serves any number of calls.  Two
+ *                   calls that may overlap (different streams) need separate
+ *                   workspaces.
  */
 int aicomp_paged_decode_attn(void* out, const void* query,
                              const void* k_pool, const void* v_pool,
