@@ -1,0 +1,148 @@
+"""Chunked-prefill causal attention through the C ABI vs the float64 oracle."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from aicomp_amd import ops, workloads
+from oracle import paged_kv_oracle as orc
+from helpers import NAME, assert_close_attn, raw, to_f64
+
+pytestmark = pytest.mark.gpu
+BF16_ATOL, BF16_RTOL = 1e-2, 2e-2
+
+
+def build_case(device, priors, news, hq, hkv, d, bs=16, dtype=torch.bfloat16, kv_dtype=None, seed=0,
+               poison=True):
+    """Random pool + table for sequences with the given prior and chunk lengths."""
+    kv_dtype = kv_dtype or dtype
+    g = torch.Generator().manual_seed(seed)
+    ctx = [p + n for p, n in zip(priors, news)]
+    need = [max(1, math.ceil(c / bs)) for c in ctx]
+    nb = sum(need) + 7
+    perm = torch.randperm(nb, generator=g)
+    table = torch.zeros(len(ctx), max(need), dtype=torch.int32)
+    cur = 0
+    for s, k in enumerate(need):
+        table[s, :k] = perm[cur:cur + k].to(torch.int32)
+        cur += k
+    T = sum(news)
+    q = torch.randn(T, hq, d, generator=g).to(dtype)
+    kf = (torch.randn(nb, hkv, bs, d, generator=g) * 0.5)
+    vf = (torch.randn(nb, hkv, bs, d, generator=g) * 0.5)
+    ks = vs = None
+    if kv_dtype == torch.float8_e4m3fn:
+        ks = (kf.abs().amax(dim=(0, 2, 3)) / 448).float()
+        vs = (vf.abs().amax(dim=(0, 2, 3)) / 448).float()
+        k_pool = (kf / ks[None, :, None, None]).to(kv_dtype)
+        v_pool = (vf / vs[None, :, None, None]).to(kv_dtype)
+    else:
+        k_pool, v_pool = kf.to(kv_dtype), vf.to(kv_dtype)
+        if poison and kv_dtype != torch.float32:
+            # every slot at or beyond a sequence's context is non-finite
+            used = torch.zeros(nb * bs, dtype=torch.bool)
+            for s, c in enumerate(ctx):
+                t = torch.arange(c)
+                used[table[s, t // bs].long() * bs + t % bs] = True
+            kflat = k_pool.permute(0, 2, 1, 3).reshape(nb * bs, hkv, d).clone()
+            vflat = v_pool.permute(0, 2, 1, 3).reshape(nb * bs, hkv, d).clone()
+            kflat[~used] = float("nan")
+            vflat[~used] = float("inf")
+            k_pool = kflat.reshape(nb, bs, hkv, d).permute(0, 2, 1, 3).contiguous()
+            v_pool = vflat.reshape(nb, bs, hkv, d).permute(0, 2, 1, 3).contiguous()
+    cu = torch.tensor([0] + list(np.cumsum(news)), dtype=torch.int32)
+    dev = lambda t: None if t is None else t.to(device)
+    return dict(q=dev(q), k_pool=dev(k_pool), v_pool=dev(v_pool), table=dev(table),
+                ctx=dev(torch.tensor(ctx, dtype=torch.int32)), cu=dev(cu), ks=dev(ks), vs=dev(vs),
+                scale=1 / math.sqrt(d), news=news, ctx_list=ctx)
+
+
+def oracle(c):
+    kp = torch.nan_to_num(c["k_pool"].float().cpu(), nan=0.0, posinf=0.0).to(c["k_pool"].dtype)
+    vp = torch.nan_to_num(c["v_pool"].float().cpu(), nan=0.0, posinf=0.0).to(c["v_pool"].dtype)
+    return orc.paged_prefill_attn(raw(c["q"]), raw(kp), raw(vp), c["table"].cpu().numpy(), c["ctx_list"],
+                                  c["cu"].cpu().numpy(), c["scale"], NAME[c["q"].dtype],
+                                  NAME[c["k_pool"].dtype],
+                                  None if c["ks"] is None else c["ks"].cpu().numpy(),
+                                  None if c["vs"] is None else c["vs"].cpu().numpy())
+
+
+def run(c, max_q_len=None):
+    out = torch.full_like(c["q"], float("nan"))
+    ops.paged_prefill_attn(out, c["q"], c["k_pool"], c["v_pool"], c["table"], c["ctx"], c["cu"],
+                           c["scale"], max_q_len=max_q_len, k_scale=c["ks"], v_scale=c["vs"])
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("hq,hkv", [(8, 2), (4, 4), (16, 2), (6, 2), (16, 1)])
+def test_prefill_small_ragged(device, hq, hkv):
+    """Ragged chunks: prior 0, prior inside a block, chunk of 1, chunk crossing tiles."""
+    c = build_case(device, priors=[0, 5, 37, 200, 0, 63], news=[70, 1, 33, 17, 1, 130], hq=hq, hkv=hkv, d=128)
+    got = to_f64(run(c, max_q_len=130))
+    assert_close_attn(got, oracle(c), BF16_ATOL, BF16_RTOL, f"{hq}/{hkv}")
+
+
+def test_prefill_reductions(device):
+    c = build_case(device, priors=[0, 300], news=[96, 1], hq=8, hkv=2, d=128, poison=False)
+    got = run(c)
+    # prior 0: torch's is_causal=True on the gathered K/V, the reference's prefill call
+    L = 96
+    blocks = c["table"][0, : L // 16].long()
+    k = c["k_pool"][blocks].permute(1, 0, 2, 3).reshape(2, L, 128).float().cpu()
+    v = c["v_pool"][blocks].permute(1, 0, 2, 3).reshape(2, L, 128).float().cpu()
+    q = c["q"][:L].float().cpu().permute(1, 0, 2)[None]
+    want = torch.nn.functional.scaled_dot_product_attention(
+        q, k.repeat_interleave(4, 0)[None], v.repeat_interleave(4, 0)[None], is_causal=True)
+    assert_close_attn(to_f64(got[:L]), want[0].permute(1, 0, 2).double().numpy(), BF16_ATOL, BF16_RTOL, "causal")
+    # chunk of one token: the decode kernel on the same sequence
+    out_d = torch.empty(1, 8, 128, dtype=torch.bfloat16, device=device)
+    ops.paged_decode_attn(out_d, c["q"][L:L + 1], c["k_pool"], c["v_pool"], c["table"][1:2].contiguous(),
+                          c["ctx"][1:2].contiguous(), c["scale"])
+    assert (out_d[0].float() - got[L].float()).abs().max() <= 2e-3
+
+
+def test_prefill_fp32_and_other_shapes_use_the_generic_kernel(device):
+    c = build_case(device, priors=[0, 9], news=[20, 7], hq=4, hkv=2, d=64, bs=8, dtype=torch.float32)
+    got = to_f64(run(c))
+    assert np.abs(got - oracle(c)).max() <= 1e-5
+
+
+def test_prefill_fp8_kv(device):
+    c = build_case(device, priors=[0, 100], news=[64, 40], hq=16, hkv=2, d=128, kv_dtype=torch.float8_e4m3fn)
+    got = to_f64(run(c))
+    assert_close_attn(got, oracle(c), BF16_ATOL, BF16_RTOL, "fp8 prefill")
+
+
+def test_config4_chunked_prefill_reduced(device):
+    """4 chunks of 512 new tokens, prior uniform in [0,2048], 32/8 heads: the named shape with the
+    decode tail cut to 2 sequences; append of all new rows first (bit-exact), then prefill."""
+    s = workloads.SHAPES["chunked_prefill_mixed"]
+    w = workloads.make_workload("x", device=device, shape=workloads.Shape(**{**s.__dict__, "batch": 2}))
+    ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping)
+    sm, bs = w.slot_mapping, 16
+    assert torch.equal(w.k_pool[sm // bs, :, sm % bs, :].view(torch.int16), w.new_key.view(torch.int16))
+    npre = w.num_prefill_seqs
+    T = int(w.cu_q_lens[npre])
+    out = torch.empty(T, 32, 128, dtype=torch.bfloat16, device=device)
+    ops.paged_prefill_attn(out, w.query[:T].contiguous(), w.k_pool, w.v_pool,
+                           w.block_table[:npre].contiguous(), w.context_lens[:npre].contiguous(),
+                           w.cu_q_lens[:npre + 1].contiguous(), w.scale, max_q_len=512)
+    torch.cuda.synchronize()
+    # oracle on a sample of rows of every chunk (first, last, tile boundaries, random)
+    rng = np.random.default_rng(0)
+    kp, vp, tab = raw(w.k_pool), raw(w.v_pool), w.block_table.cpu().numpy()
+    qraw = raw(w.query)
+    got = to_f64(out)
+    for sidx in range(npre):
+        n, L = w.new_list[sidx], w.ctx_list[sidx]
+        prior = L - n
+        rows = sorted(set([0, 1, 15, 16, 63, 64, 255, 511] + rng.integers(0, n, 6).tolist()))
+        k = orc.decode_elements(orc.gather_context(kp, tab[sidx], L), "bf16")
+        v = orc.decode_elements(orc.gather_context(vp, tab[sidx], L), "bf16")
+        for i in rows:
+            r = int(w.cu_q_lens[sidx]) + i
+            qv = orc.decode_elements(qraw[r], "bf16")[None]
+            want = orc.attend_contiguous(qv, k[: prior + i + 1], v[: prior + i + 1], w.scale)[0]
+            assert_close_attn(got[r], want, BF16_ATOL, BF16_RTOL, f"chunk {sidx} row {i}")
