@@ -1,0 +1,56 @@
+"""The C-ABI library loads and exports every function include/aicomp_kv.h declares
+(no compute calls: this runs without a GPU)."""
+import ctypes
+import os
+import re
+
+from aicomp_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "aicomp_kv.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(aicomp_\w+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    names = declared_functions()
+    assert names, "no declarations found"
+    assert sorted(_lib.SYMBOLS) == names
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} missing from {_lib.LIB_PATH}"
+
+
+def test_host_only_entry_points():
+    lib = _lib.load()
+    assert lib.aicomp_kv_version() >= 100
+    # sizing helpers are pure host arithmetic
+    ps = lib.aicomp_paged_decode_partition_size(64, 32, 8, 128, 16, 257, _lib.BF16, _lib.BF16)
+    assert ps > 0 and ps % 16 == 0
+    need = lib.aicomp_paged_decode_workspace_bytes(64, 32, 8, 128, 16, 257, _lib.BF16, _lib.BF16, 0)
+    parts = -(-257 * 16 // ps)
+    assert need == (64 * 8 * 4 + 255) // 256 * 256 + 64 * 32 * parts * (128 + 2) * 4
+    assert lib.aicomp_paged_decode_workspace_bytes(4, 8, 2, 128, 16, 4, _lib.BF16, _lib.BF16, 64) == 0
+    # argument validation happens before any device work
+    rc = lib.aicomp_paged_decode_attn(None, None, None, None, None, 0, None, 4, 8, 2, 128, 16, 4, 16,
+                                      1.0, _lib.BF16, _lib.BF16, None, None, 0, None, 0, None)
+    assert rc == 1 and b"null pointer" in lib.aicomp_kv_last_error()
+    rc = lib.aicomp_kv_append(None, None, 0, 0, None, None, None, -1, 1, 1, 1, 1, 0, 0, None, None, None)
+    assert rc == 1
+    assert lib.aicomp_kv_append(None, None, 0, 0, None, None, None, 0, 1, 1, 1, 1, 0, 0, None, None, None) == 0
+
+
+def test_ops_refuse_cpu_tensors():
+    import pytest
+    import torch
+    from aicomp_amd import ops
+    k = torch.zeros(2, 1, 16, 64, dtype=torch.bfloat16)
+    x = torch.zeros(1, 1, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError):
+        ops.kv_append(x, x, k, k, torch.zeros(1, dtype=torch.int64))
