@@ -101,16 +101,26 @@ static int resolve_parts(int64_t rows, int hkv, int bs, int max_blocks, int& par
     return (int)(parts < 1 ? 1 : parts);
 }
 
+static bool streamk_shape(int batch, int hq, int hkv, int d, int bs, int q_dtype, int kv_dtype) {
+    return d == 128 && bs == 16 && q_dtype == AICOMP_KV_BF16 &&
+           (kv_dtype == AICOMP_KV_BF16 || kv_dtype == AICOMP_KV_FP8_E4M3) && hq / hkv <= 16 &&
+           batch <= 1024;
+}
+
 size_t aicomp_paged_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads,
                                            int head_dim, int block_size, int max_blocks_per_seq,
                                            int q_dtype, int kv_dtype, int partition_size) {
-    (void)q_dtype; (void)kv_dtype;
     if (batch <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || block_size <= 0 ||
-        max_blocks_per_seq <= 0)
+        max_blocks_per_seq <= 0 || num_q_heads % num_kv_heads)
         return 0;
+    const bool automatic = partition_size <= 0;
     const int parts = resolve_parts(batch, num_kv_heads, block_size, max_blocks_per_seq, partition_size);
-    if (parts <= 1) return 0;
-    return split_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, parts);
+    size_t need = parts <= 1 ? 0 : split_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, parts);
+    if (automatic && streamk_shape(batch, num_q_heads, num_kv_heads, head_dim, block_size, q_dtype, kv_dtype)) {
+        const size_t sk = decode_streamk_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim);
+        if (sk > need) need = sk;
+    }
+    return need;
 }
 
 int aicomp_paged_decode_attn(void* out, const void* query, const void* k_pool, const void* v_pool,
@@ -148,6 +158,16 @@ int aicomp_paged_decode_attn(void* out, const void* query, const void* k_pool, c
     a.partition_size = partition_size;
     a.num_parts = resolve_parts(batch, num_kv_heads, block_size, max_blocks_per_seq, a.partition_size);
     a.stream = (hipStream_t)stream;
+    if (partition_size == 0 && decode_streamk_supported(a)) {
+        // balanced schedule: equal tile counts per wave, merged by a second kernel
+        const size_t need = decode_streamk_workspace_bytes(a.rows, a.hq, a.hkv, a.d);
+        AICOMP_REQUIRE(workspace && workspace_bytes >= need, AICOMP_KV_EWORKSPACE,
+                       "paged_decode_attn: workspace of %zu bytes needed, %zu given", need,
+                       workspace ? workspace_bytes : (size_t)0);
+        AICOMP_REQUIRE((uintptr_t)workspace % 16 == 0, AICOMP_KV_EINVAL,
+                       "paged_decode_attn: workspace must be 16-byte aligned");
+        return launch_decode_streamk(a, workspace);
+    }
     if (a.num_parts > 1) {
         const size_t need = split_workspace_bytes(a.rows, a.hq, a.hkv, a.d, a.num_parts);
         AICOMP_REQUIRE(workspace && workspace_bytes >= need, AICOMP_KV_EWORKSPACE,

@@ -157,6 +157,9 @@ struct DecodeArgs {
 int launch_decode_generic(const DecodeArgs& a);
 bool decode_mfma_supported(const DecodeArgs& a);
 int launch_decode_mfma(const DecodeArgs& a);
+bool decode_streamk_supported(const DecodeArgs& a);
+size_t decode_streamk_workspace_bytes(int64_t rows, int hq, int hkv, int d);
+int launch_decode_streamk(const DecodeArgs& a, void* workspace);
 int launch_split_reduce(const DecodeArgs& a);
 
 }  // namespace aicomp

@@ -38,6 +38,7 @@
 //              last partition (device-scope counter) merges them in the same
 //              launch, so a decode call is one kernel.
 #include "common.h"
+#include <stdlib.h>
 
 namespace aicomp {
 
@@ -54,6 +55,7 @@ constexpr int NWAVES = 4;
 constexpr int KROW = 272;              // LDS row stride in bytes (256 + 16 pad)
 constexpr int KTILE_BYTES = TILE * KROW;   // 8704 per wave
 constexpr float NEG_BIG = -1.0e30f;
+constexpr int SK_MAX_WAVES = 4096;     // balanced schedule: at most 1024 workgroups of 4 waves
 
 struct MfmaParams {
     void* out;
@@ -235,10 +237,7 @@ __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, T
 }
 
 template <bool FP8>
-#ifndef EXP_WPS
-#define EXP_WPS 2
-#endif
-__global__ void __launch_bounds__(256, EXP_WPS)
+__global__ void __launch_bounds__(256, 2)
 paged_decode_mfma_kernel(MfmaParams p) {
     // KV head fastest: the workgroups launched together read the Hkv slices of the same
     // physical blocks, i.e. one contiguous Hkv*4 KB piece of each pool
@@ -341,10 +340,6 @@ paged_decode_mfma_kernel(MfmaParams p) {
     const float m = st.m;
     float lsum = st.lsum;
     f32x4_t (&O)[8] = st.O;
-#ifdef EXP_NO_EPI
-    if (p.num_parts == 12345) ((float*)p.out)[tid] = m + lsum + O[0][0] + O[1][1] + O[2][2] + O[3][3] + O[4][0] + O[5][1] + O[6][2] + O[7][3];
-    return;
-#endif
 
     // ---- wave result: lane (head r16, g4) holds O^T[dim 32*g4 + 8*i + j][head] in O[j][i]
     lsum += __shfl_xor(lsum, 16);
@@ -390,6 +385,281 @@ paged_decode_mfma_kernel(MfmaParams p) {
     }
 }
 
+
+// ---------------------------------------------------------------------------------------
+// Balanced schedule.  The grid above gives the hardware dispatcher workgroups of unequal
+// size and leaves a tail where few of them are still streaming.  Here the launch is
+// exactly one workgroup per CU and every WAVE gets the same number of 32-token tiles:
+// the tiles of all (sequence, KV head) rows form one sequence (row-major, KV head inside
+// sequence), wave i owns tiles [i*N/W, (i+1)*N/W).  A wave crossing a row boundary flushes
+// its partial (max, sum, unnormalised output) and starts the next row, so all waves start
+// together, stream the same number of bytes and finish together.  Partials go to slot
+// (wave index + row index) - strictly increasing along the schedule, hence unique - and
+// streamk_reduce_kernel merges the slots of each row.  No barrier after the prologue.
+constexpr int SK_MAX_SEQS = 1024;
+
+struct StreamKParams {
+    void* out;
+    const void* query;
+    const void* k_pool;
+    const void* v_pool;
+    const int32_t* block_table;
+    int64_t block_table_stride;
+    const int32_t* context_lens;
+    int num_seqs, hq, hkv, group, max_blocks;
+    int64_t num_blocks;
+    float qk_mul;
+    const float* k_scale;
+    const float* v_scale;
+    int num_waves;
+    float* ws_acc;      // [slots][G][D]
+    float* ws_ml;       // [slots][G][2]
+};
+
+__device__ __forceinline__ int sk_tiles(int len, int max_blocks) {
+    len = min(max(len, 0), max_blocks * BS);
+    return (len + TILE - 1) / TILE;
+}
+
+// wave that owns global tile g when N tiles are dealt to W waves as [i*N/W, (i+1)*N/W)
+__device__ __forceinline__ int sk_wave_of(int64_t g, int64_t N, int W) {
+    return (int)(((g + 1) * W - 1) / N);
+}
+
+template <bool FP8>
+__global__ void __launch_bounds__(256, 2)
+streamk_decode_kernel(StreamKParams p) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, g4 = lane >> 4;
+    const int G = p.group, B = p.num_seqs;
+
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NWAVES * KTILE_BYTES];
+    __shared__ int prefix[SK_MAX_SEQS + 1];     // prefix[s] = tiles of the sequences before s
+    __shared__ int wave_tot[NWAVES];
+    unsigned char* kt = lds + w * KTILE_BYTES;
+
+    // ---- prologue: tiles per sequence -> exclusive prefix sums (4 sequences per thread)
+    {
+        int loc[4], sum = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int sidx = 4 * tid + k;
+            loc[k] = sidx < B ? sk_tiles(p.context_lens[sidx], p.max_blocks) : 0;
+            sum += loc[k];
+        }
+        int inc = sum;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int v = __shfl_up(inc, o);
+            if (lane >= o) inc += v;
+        }
+        if (lane == 63) wave_tot[w] = inc;
+        __syncthreads();
+        int base = inc - sum;
+        for (int ww = 0; ww < w; ++ww) base += wave_tot[ww];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int sidx = 4 * tid + k;
+            if (sidx <= B) prefix[sidx] = base;
+            base += loc[k];
+        }
+        if (tid == 255 && B == SK_MAX_SEQS) prefix[SK_MAX_SEQS] = base;
+        __syncthreads();
+    }
+    const int64_t N = (int64_t)p.hkv * __builtin_amdgcn_readfirstlane(prefix[B]);
+    const int wave_id = blockIdx.x * NWAVES + w;
+    const int W = (int)min((int64_t)p.num_waves, N);      // with fewer tiles than waves, one tile each
+    if (wave_id >= W) return;
+    const int64_t g0 = (int64_t)wave_id * N / W;
+    const int64_t g1 = (int64_t)(wave_id + 1) * N / W;
+
+    // ---- first row of this wave: largest s with prefix[s] <= g0 / Hkv
+    int seq;
+    {
+        const int x = (int)(g0 / p.hkv);
+        int lo = 0, hi = B;            // invariant: prefix[lo] <= x < prefix[hi]
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (prefix[mid] <= x) lo = mid; else hi = mid;
+        }
+        seq = __builtin_amdgcn_readfirstlane(lo);
+    }
+    // everything that steers the loop is wave-uniform: keep it in scalar registers
+    int row_tiles = __builtin_amdgcn_readfirstlane(prefix[seq + 1] - prefix[seq]);
+    int kvh, t;
+    {
+        const int rem = (int)(g0 - (int64_t)p.hkv * prefix[seq]);
+        kvh = __builtin_amdgcn_readfirstlane(rem / row_tiles);
+        t = __builtin_amdgcn_readfirstlane(rem % row_tiles);
+    }
+
+    const int wr_off = (lane >> 4) * KROW + (lane & 15) * 16;
+    const int rd_off = (4 * (r16 & 3) + (r16 >> 2)) * KROW + g4 * 16;
+
+    for (int64_t g = g0; g < g1 && seq < B;) {
+        const int nt = (int)min((int64_t)(row_tiles - t), g1 - g);       // tiles of this segment (>= 1)
+        const int len = min(p.context_lens[seq], p.max_blocks * BS);
+
+        // Q rows and the table slice of the segment, one wait for both
+        const int32_t* table = p.block_table + (int64_t)seq * p.block_table_stride;
+        const int blk_base = 2 * t;
+        int tab_first = 0;
+        int tab = (blk_base + lane < p.max_blocks) ? table[blk_base + lane] : 0;
+        bf16x8_t qf[4];
+        {
+            const uint4* qp = (const uint4*)((const bf16_t*)p.query +
+                                             ((int64_t)seq * p.hq + kvh * G + min(r16, G - 1)) * D + 8 * g4);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                uint4 v = qp[s * 4];
+                if (r16 >= G) v = make_uint4(0, 0, 0, 0);
+                qf[s] = __builtin_bit_cast(bf16x8_t, v);
+            }
+        }
+        const float cmul = p.qk_mul * (FP8 ? p.k_scale[kvh] : 1.f);
+        auto tile_blocks = [&](int k, int64_t& b0, int64_t& b1) {      // k-th tile of the segment
+            const int i0 = 2 * k;
+            if (i0 - tab_first >= 64) {
+                tab_first = i0;
+                tab = (blk_base + i0 + lane < p.max_blocks) ? table[blk_base + i0 + lane] : 0;
+                __builtin_amdgcn_s_waitcnt(0x0F70);
+            }
+            b0 = clamp_block(__builtin_amdgcn_readlane(tab, i0 - tab_first), p.num_blocks);
+            b1 = clamp_block(__builtin_amdgcn_readlane(tab, i0 + 1 - tab_first), p.num_blocks);
+        };
+
+        WaveState st;
+        st.m = NEG_BIG; st.lsum = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) st.O[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+        TileRegs<FP8> kr, vr;
+        int64_t b0, b1;
+        __builtin_amdgcn_s_waitcnt(0x0F70);          // Q and table have landed
+        tile_blocks(0, b0, b1);
+        load_tile<FP8>(kr, p.k_pool, b0, b1, p.hkv, kvh, lane);
+        load_tile<FP8>(vr, p.v_pool, b0, b1, p.hkv, kvh, lane);
+        int k = 0;
+        for (; k + 1 < nt; ++k) {
+            tile_blocks(k + 1, b0, b1);
+            process_tile<FP8, true, false>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, b0, b1,
+                                           p.hkv, kvh, lane, g4, (t + k) * TILE, len, cmul);
+        }
+        const int tile_start = (t + k) * TILE;
+        if (tile_start + TILE > len)
+            process_tile<FP8, false, true>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
+                                           p.hkv, kvh, lane, g4, tile_start, len, cmul);
+        else
+            process_tile<FP8, false, false>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
+                                            p.hkv, kvh, lane, g4, tile_start, len, cmul);
+
+        // ---- flush: lane (head r16, g4) holds O^T[dim 32*g4 + 8*i + j][head] in O[j][i]
+        float lsum = st.lsum;
+        lsum += __shfl_xor(lsum, 16);
+        lsum += __shfl_xor(lsum, 32);
+        if (r16 < G) {
+            const int64_t slot = (int64_t)wave_id + ((int64_t)seq * p.hkv + kvh);
+            float* dst = p.ws_acc + (slot * G + r16) * D + 32 * g4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                *(float4*)(dst + 8 * i) = make_float4(st.O[0][i], st.O[1][i], st.O[2][i], st.O[3][i]);
+                *(float4*)(dst + 8 * i + 4) = make_float4(st.O[4][i], st.O[5][i], st.O[6][i], st.O[7][i]);
+            }
+            if (g4 == 0) *(float2*)(p.ws_ml + (slot * G + r16) * 2) = make_float2(st.m, lsum);
+        }
+
+        // ---- next row
+        g += nt;
+        t = 0;
+        if (++kvh == p.hkv) {
+            kvh = 0;
+            do { ++seq; } while (seq < B && __builtin_amdgcn_readfirstlane(prefix[seq + 1] - prefix[seq]) == 0);
+            if (seq < B) row_tiles = __builtin_amdgcn_readfirstlane(prefix[seq + 1] - prefix[seq]);
+        }
+    }
+}
+
+// Merge of the balanced schedule's partials: one workgroup per (KV head, sequence, head of
+// the group).  The row's partials sit in consecutive slots first+row .. last+row; their
+// weights 2^(m_i - M) are computed once (one lane per partial) and parked in LDS, then each
+// lane accumulates one output dim with independent loads.
+constexpr int SK_RED_CACHE = 512;
+
+__global__ void __launch_bounds__(128)
+streamk_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws_acc,
+                      const float* __restrict__ ws_ml, const int32_t* __restrict__ context_lens,
+                      int num_seqs, int hq, int hkv, int group, int max_blocks, int num_waves,
+                      const float* __restrict__ v_scale) {
+    const int kvh = blockIdx.x, seq = blockIdx.y, h = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    __shared__ int redi[2][2];
+    __shared__ float redf[2][2];
+    __shared__ float wgt[SK_RED_CACHE];
+    // tiles before this sequence, and in total
+    int before = 0, total = 0;
+    for (int sidx = tid; sidx < num_seqs; sidx += 128) {
+        const int tl = sk_tiles(context_lens[sidx], max_blocks);
+        total += tl;
+        if (sidx < seq) before += tl;
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) { before += __shfl_xor(before, o); total += __shfl_xor(total, o); }
+    if (lane == 0) { redi[0][wv] = before; redi[1][wv] = total; }
+    __syncthreads();
+    before = redi[0][0] + redi[0][1];
+    total = redi[1][0] + redi[1][1];
+    const int row_tiles = sk_tiles(context_lens[seq], max_blocks);
+    bf16_t* o = out + ((int64_t)seq * hq + kvh * group + h) * D;
+    if (row_tiles == 0) {
+        o[tid].bits = 0;
+        return;
+    }
+    const int64_t N = (int64_t)hkv * total;
+    const int W = (int)min((int64_t)num_waves, N);        // every one of the W waves owns >= 1 tile
+    const int64_t gr = (int64_t)hkv * before + (int64_t)kvh * row_tiles;
+    const int first = sk_wave_of(gr, N, W);
+    const int last = sk_wave_of(gr + row_tiles - 1, N, W);
+    const int np = last - first + 1;
+    const int64_t row = (int64_t)seq * hkv + kvh;
+    const float* ml = ws_ml + ((first + row) * group + h) * 2;          // partial i at ml[i * group * 2]
+    const float* acc = ws_acc + ((first + row) * group + h) * D + tid;  // partial i at acc[i * group * D]
+    float mx = NEG_BIG;
+    for (int i = tid; i < np; i += 128) mx = fmaxf(mx, ml[(int64_t)i * group * 2]);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+    if (lane == 0) redf[0][wv] = mx;
+    __syncthreads();
+    mx = fmaxf(redf[0][0], redf[0][1]);
+    float den = 0.f;
+    for (int i = tid; i < np; i += 128) {
+        const float f = exp2f(ml[(int64_t)i * group * 2] - mx);
+        if (i < SK_RED_CACHE) wgt[i] = f;
+        den = fmaf(f, ml[(int64_t)i * group * 2 + 1], den);
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) den += __shfl_xor(den, off);
+    if (lane == 0) redf[1][wv] = den;
+    __syncthreads();
+    den = redf[1][0] + redf[1][1];
+    const int64_t stride = (int64_t)group * D;
+    float num = 0.f;
+    int i = 0;
+    for (; i + 4 <= np && i + 4 <= SK_RED_CACHE; i += 4) {
+        const float a0 = acc[i * stride], a1 = acc[(i + 1) * stride];
+        const float a2 = acc[(i + 2) * stride], a3 = acc[(i + 3) * stride];
+        num = fmaf(wgt[i], a0, num); num = fmaf(wgt[i + 1], a1, num);
+        num = fmaf(wgt[i + 2], a2, num); num = fmaf(wgt[i + 3], a3, num);
+    }
+    for (; i < np; ++i) {
+        const float f = i < SK_RED_CACHE ? wgt[i] : exp2f(ml[(int64_t)i * group * 2] - mx);
+        num = fmaf(f, acc[i * stride], num);
+    }
+    const float vs = v_scale ? v_scale[kvh] : 1.f;
+    o[tid].bits = f32_to_bf16(den > 0.f ? vs * num / den : 0.f);
+}
+
 }  // namespace
 
 bool decode_mfma_supported(const DecodeArgs& a) {
@@ -399,6 +669,55 @@ bool decode_mfma_supported(const DecodeArgs& a) {
            group <= 16 && a.scale > 0.f && a.partition_size % TILE == 0 && a.rows <= 65535 &&
            a.num_parts <= 65535 && ((uintptr_t)a.query % 16 == 0) && ((uintptr_t)a.k_pool % 16 == 0) &&
            ((uintptr_t)a.v_pool % 16 == 0);
+}
+
+bool decode_streamk_supported(const DecodeArgs& a) {
+    return decode_mfma_supported(a) && a.rows <= SK_MAX_SEQS;
+}
+
+size_t decode_streamk_workspace_bytes(int64_t rows, int hq, int hkv, int d) {
+    const int64_t slots = SK_MAX_WAVES + rows * hkv;
+    return (size_t)slots * (hq / hkv) * (size_t)(d + 2) * sizeof(float);
+}
+
+int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
+    static int num_cus = 0;
+    if (num_cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            set_error("paged_decode_attn: cannot query the CU count");
+            return AICOMP_KV_EHIP;
+        }
+        num_cus = n;
+    }
+    // one workgroup per CU measured fastest (4 waves of 16 KB in flight each already cover the
+    // HBM latency; a second workgroup per CU only adds partials and start-up work)
+    int wgs = min(num_cus, SK_MAX_WAVES / NWAVES);
+    if (const char* e = getenv("AICOMP_SK_WGS")) wgs = min(atoi(e), SK_MAX_WAVES / NWAVES);  // EXPERIMENT
+    const int group = a.hq / a.hkv;
+    const int64_t slots = SK_MAX_WAVES + a.rows * a.hkv;
+    StreamKParams p;
+    p.out = a.out; p.query = a.query; p.k_pool = a.k_pool; p.v_pool = a.v_pool;
+    p.block_table = a.block_table; p.block_table_stride = a.block_table_stride;
+    p.context_lens = a.context_lens;
+    p.num_seqs = (int)a.rows; p.hq = a.hq; p.hkv = a.hkv; p.group = group; p.max_blocks = a.max_blocks;
+    p.num_blocks = a.num_blocks;
+    p.qk_mul = a.scale * LOG2E;
+    p.k_scale = a.k_scale; p.v_scale = a.v_scale;
+    p.num_waves = wgs * NWAVES;
+    p.ws_acc = (float*)workspace;
+    p.ws_ml = p.ws_acc + slots * group * D;
+    if (a.kv_dtype == AICOMP_KV_FP8_E4M3)
+        hipLaunchKernelGGL(streamk_decode_kernel<true>, dim3(wgs), dim3(256), 0, a.stream, p);
+    else
+        hipLaunchKernelGGL(streamk_decode_kernel<false>, dim3(wgs), dim3(256), 0, a.stream, p);
+    AICOMP_HIP_LAUNCH_CHECK();
+    hipLaunchKernelGGL(streamk_reduce_kernel, dim3(a.hkv, (unsigned)a.rows, group), dim3(128), 0, a.stream,
+                       (bf16_t*)a.out, p.ws_acc, p.ws_ml, a.context_lens, (int)a.rows, a.hq, a.hkv, group,
+                       a.max_blocks, p.num_waves, a.v_scale);
+    AICOMP_HIP_LAUNCH_CHECK();
+    return AICOMP_KV_OK;
 }
 
 int launch_decode_mfma(const DecodeArgs& a) {

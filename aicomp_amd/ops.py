@@ -125,6 +125,7 @@ def paged_decode_attn(out: torch.Tensor, query: torch.Tensor, k_pool: torch.Tens
     ``context_lens [B]`` int32.  In place on ``out``, on the current stream.
     """
     lib = _lib.load()
+    _req(query.is_cuda, "tensors must live on a ROCm device (there is no CPU path)")
     nb, hkv, bs, d = _check_pools(k_pool, v_pool)
     _req(query.dim() == 3 and out.shape == query.shape and out.dtype == query.dtype,
          f"out/query must both be [B, Hq, D]; got {tuple(out.shape)} and {tuple(query.shape)}")
