@@ -26,8 +26,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 METRIC = "decode-attn HBM GB/s (% peak) + tokens/s, Llama-3-8B paged KV, 1 GPU"
 
 # HBM bytes per decode launch of the Llama-3-8B shape from rocprofv3 --pmc
-# (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); None until measured.
-MEASURED_TRAFFIC_BYTES = None
+# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, the factors a 1 GiB device copy gives), main + merge kernel.
+MEASURED_TRAFFIC_BYTES = 651.9e6   # profiles/decode_llama3_8b_decode.md
 
 
 def _events(n):
@@ -62,7 +62,7 @@ def run_decode_config(name, steps, warmup, dev):
         if ev: ev[1].record()
         if npre:
             ops.paged_prefill_attn(outp, qp, w.k_pool, w.v_pool, btp, clp, cup, w.scale, max_q_len=max_q)
-        if ev: ev[2].record()
+            if ev: ev[2].record()
         ops.paged_decode_attn(outd, qd, w.k_pool, w.v_pool, btd, cld, w.scale, w.k_scale, w.v_scale)
         if ev: ev[3].record()
 
@@ -73,13 +73,15 @@ def run_decode_config(name, steps, warmup, dev):
     t0 = time.perf_counter()
     for i in range(steps):
         step(evs[i])
+    t_enqueue = time.perf_counter() - t0
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     t_app = statistics.mean(e[0].elapsed_time(e[1]) for e in evs) * 1e-3
-    t_pre = statistics.mean(e[1].elapsed_time(e[2]) for e in evs) * 1e-3
-    t_dec = statistics.mean(e[2].elapsed_time(e[3]) for e in evs) * 1e-3
+    t_pre = statistics.mean(e[1].elapsed_time(e[2]) for e in evs) * 1e-3 if npre else 0.0
+    t_dec = statistics.mean(e[2 if npre else 1].elapsed_time(e[3]) for e in evs) * 1e-3
     res = {
         "workload": name, "ms_per_step": wall / steps * 1e3,
+        "host_enqueue_ms_per_step": t_enqueue / steps * 1e3,
         "append_us": t_app * 1e6, "append_bytes": w.append_bytes(),
         "append_GBs": w.append_bytes() / t_app / 1e9,
         "decode_us": t_dec * 1e6, "decode_bytes": w.decode_kv_bytes(),
@@ -233,7 +235,7 @@ def main():
                    "kv_bytes_per_step": main_res["decode_bytes"]},
         "tokens_per_s": s.batch / (main_res["ms_per_step"] * 1e-3),
         "pct_hbm_peak": 100.0 * main_res["decode_bytes"] / (main_res["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
-        "roofline": {"kernel": "paged_decode_mfma_kernel<bf16> + split_reduce_kernel (one decode call)",
+        "roofline": {"kernel": "streamk_decode_kernel<bf16> + streamk_reduce_kernel (one decode call)",
                      "bound": "hbm", "achieved": main_res["decode_GBs"], "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": main_res["decode_GBs"] / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES,
