@@ -123,27 +123,31 @@ size_t aicomp_paged_decode_workspace_bytes(int batch, int num_q_heads, int num_k
     return need;
 }
 
-int aicomp_paged_decode_attn(void* out, const void* query, const void* k_pool, const void* v_pool,
-                             const int32_t* block_table, int64_t block_table_stride,
-                             const int32_t* context_lens, int batch, int num_q_heads,
-                             int num_kv_heads, int head_dim, int block_size,
-                             int max_blocks_per_seq, int64_t num_blocks, float scale, int q_dtype,
-                             int kv_dtype, const float* k_scale, const float* v_scale,
-                             int partition_size, void* workspace, size_t workspace_bytes,
-                             void* stream) {
-    AICOMP_REQUIRE(batch >= 0, AICOMP_KV_EINVAL, "paged_decode_attn: negative batch");
+static int decode_impl(void* out, const void* query, const void* new_key, const void* new_value,
+                       int64_t kv_token_stride, int64_t kv_head_stride, void* k_pool, void* v_pool,
+                       const int32_t* block_table, int64_t block_table_stride,
+                       const int32_t* context_lens, int batch, int num_q_heads, int num_kv_heads,
+                       int head_dim, int block_size, int max_blocks_per_seq, int64_t num_blocks,
+                       float scale, int q_dtype, int kv_dtype, const float* k_scale,
+                       const float* v_scale, int partition_size, void* workspace,
+                       size_t workspace_bytes, void* stream, const char* who) {
+    AICOMP_REQUIRE(batch >= 0, AICOMP_KV_EINVAL, "%s: negative batch", who);
     if (batch == 0) return AICOMP_KV_OK;
     AICOMP_REQUIRE(out && query && k_pool && v_pool && block_table && context_lens,
-                   AICOMP_KV_EINVAL, "paged_decode_attn: null pointer");
+                   AICOMP_KV_EINVAL, "%s: null pointer", who);
     int rc = check_common(num_q_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq,
-                          num_blocks, q_dtype, kv_dtype, k_scale, v_scale, "paged_decode_attn");
+                          num_blocks, q_dtype, kv_dtype, k_scale, v_scale, who);
     if (rc) return rc;
     AICOMP_REQUIRE(max_blocks_per_seq > 0 && block_table_stride >= max_blocks_per_seq,
-                   AICOMP_KV_EINVAL, "paged_decode_attn: block table stride %lld < width %d",
+                   AICOMP_KV_EINVAL, "%s: block table stride %lld < width %d", who,
                    (long long)block_table_stride, max_blocks_per_seq);
     AICOMP_REQUIRE(partition_size >= 0 && partition_size % block_size == 0, AICOMP_KV_EINVAL,
-                   "paged_decode_attn: partition_size %d is not a multiple of block_size %d",
-                   partition_size, block_size);
+                   "%s: partition_size %d is not a multiple of block_size %d", who, partition_size,
+                   block_size);
+    const bool fused = new_key != nullptr;
+    if (fused)
+        AICOMP_REQUIRE(new_value && kv_head_stride >= head_dim && kv_token_stride >= 0, AICOMP_KV_EINVAL,
+                       "%s: bad new_key / new_value arguments", who);
     DecodeArgs a;
     memset(&a, 0, sizeof(a));
     a.out = out; a.query = query; a.k_pool = k_pool; a.v_pool = v_pool;
@@ -162,23 +166,79 @@ int aicomp_paged_decode_attn(void* out, const void* query, const void* k_pool, c
         // balanced schedule: equal tile counts per wave, merged by a second kernel
         const size_t need = decode_streamk_workspace_bytes(a.rows, a.hq, a.hkv, a.d);
         AICOMP_REQUIRE(workspace && workspace_bytes >= need, AICOMP_KV_EWORKSPACE,
-                       "paged_decode_attn: workspace of %zu bytes needed, %zu given", need,
+                       "%s: workspace of %zu bytes needed, %zu given", who, need,
                        workspace ? workspace_bytes : (size_t)0);
         AICOMP_REQUIRE((uintptr_t)workspace % 16 == 0, AICOMP_KV_EINVAL,
-                       "paged_decode_attn: workspace must be 16-byte aligned");
+                       "%s: workspace must be 16-byte aligned", who);
+        // the kernel appends the new rows itself when it can read them 16 bytes at a time
+        const bool in_kernel = fused && q_dtype == AICOMP_KV_BF16 && kv_token_stride % 8 == 0 &&
+                               kv_head_stride % 8 == 0 && (uintptr_t)new_key % 16 == 0 &&
+                               (uintptr_t)new_value % 16 == 0;
+        if (fused && !in_kernel) {
+            rc = launch_kv_append_last(new_key, new_value, kv_token_stride, kv_head_stride, k_pool, v_pool,
+                                       block_table, block_table_stride, context_lens, batch,
+                                       num_kv_heads, head_dim, block_size, max_blocks_per_seq,
+                                       num_blocks, q_dtype, kv_dtype, k_scale, v_scale, a.stream);
+            if (rc) return rc;
+        }
+        if (in_kernel) {
+            a.new_key = new_key; a.new_value = new_value;
+            a.new_token_stride = kv_token_stride; a.new_head_stride = kv_head_stride;
+        }
         return launch_decode_streamk(a, workspace);
+    }
+    if (fused) {
+        rc = launch_kv_append_last(new_key, new_value, kv_token_stride, kv_head_stride, k_pool, v_pool,
+                                   block_table, block_table_stride, context_lens, batch, num_kv_heads,
+                                   head_dim, block_size, max_blocks_per_seq, num_blocks, q_dtype,
+                                   kv_dtype, k_scale, v_scale, a.stream);
+        if (rc) return rc;
     }
     if (a.num_parts > 1) {
         const size_t need = split_workspace_bytes(a.rows, a.hq, a.hkv, a.d, a.num_parts);
         AICOMP_REQUIRE(workspace && workspace_bytes >= need, AICOMP_KV_EWORKSPACE,
-                       "paged_decode_attn: workspace of %zu bytes needed, %zu given", need,
+                       "%s: workspace of %zu bytes needed, %zu given", who, need,
                        workspace ? workspace_bytes : (size_t)0);
         AICOMP_REQUIRE((uintptr_t)workspace % 16 == 0, AICOMP_KV_EINVAL,
-                       "paged_decode_attn: workspace must be 16-byte aligned");
+                       "%s: workspace must be 16-byte aligned", who);
         a.ws = split_workspace_view(workspace, a.rows, a.hq, a.hkv, a.d, a.num_parts);
     }
     if (decode_mfma_supported(a)) return launch_decode_mfma(a);
     return launch_decode_generic(a);
+}
+
+int aicomp_paged_decode_attn(void* out, const void* query, const void* k_pool, const void* v_pool,
+                             const int32_t* block_table, int64_t block_table_stride,
+                             const int32_t* context_lens, int batch, int num_q_heads,
+                             int num_kv_heads, int head_dim, int block_size,
+                             int max_blocks_per_seq, int64_t num_blocks, float scale, int q_dtype,
+                             int kv_dtype, const float* k_scale, const float* v_scale,
+                             int partition_size, void* workspace, size_t workspace_bytes,
+                             void* stream) {
+    return decode_impl(out, query, nullptr, nullptr, 0, 0, (void*)k_pool, (void*)v_pool, block_table,
+                       block_table_stride, context_lens, batch, num_q_heads, num_kv_heads, head_dim,
+                       block_size, max_blocks_per_seq, num_blocks, scale, q_dtype, kv_dtype, k_scale,
+                       v_scale, partition_size, workspace, workspace_bytes, stream,
+                       "paged_decode_attn");
+}
+
+int aicomp_paged_decode_attn_append(void* out, const void* query, const void* new_key,
+                                    const void* new_value, int64_t kv_token_stride,
+                                    int64_t kv_head_stride, void* k_pool, void* v_pool,
+                                    const int32_t* block_table, int64_t block_table_stride,
+                                    const int32_t* context_lens, int batch, int num_q_heads,
+                                    int num_kv_heads, int head_dim, int block_size,
+                                    int max_blocks_per_seq, int64_t num_blocks, float scale,
+                                    int q_dtype, int kv_dtype, const float* k_scale,
+                                    const float* v_scale, int partition_size, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+    AICOMP_REQUIRE(batch <= 0 || (new_key && new_value), AICOMP_KV_EINVAL,
+                   "paged_decode_attn_append: null new_key / new_value");
+    return decode_impl(out, query, new_key, new_value, kv_token_stride, kv_head_stride, k_pool, v_pool,
+                       block_table, block_table_stride, context_lens, batch, num_q_heads, num_kv_heads,
+                       head_dim, block_size, max_blocks_per_seq, num_blocks, scale, q_dtype, kv_dtype,
+                       k_scale, v_scale, partition_size, workspace, workspace_bytes, stream,
+                       "paged_decode_attn_append");
 }
 
 int aicomp_paged_prefill_attn(void* out, const void* query, const void* k_pool, const void* v_pool,

@@ -152,6 +152,10 @@ struct DecodeArgs {
     int num_parts;              // ceil(max_blocks*bs / partition_size)
     SplitWorkspace ws;
     hipStream_t stream;
+    // fused append of one new token per sequence (decode only; NULL = none)
+    const void* new_key;
+    const void* new_value;
+    int64_t new_token_stride, new_head_stride;
 };
 
 int launch_decode_generic(const DecodeArgs& a);
@@ -160,6 +164,12 @@ int launch_decode_mfma(const DecodeArgs& a);
 bool decode_streamk_supported(const DecodeArgs& a);
 size_t decode_streamk_workspace_bytes(int64_t rows, int hq, int hkv, int d);
 int launch_decode_streamk(const DecodeArgs& a, void* workspace);
+int launch_kv_append_last(const void* key, const void* value, int64_t token_stride, int64_t head_stride,
+                          void* k_pool, void* v_pool, const int32_t* block_table,
+                          int64_t block_table_stride, const int32_t* context_lens, int batch, int hkv,
+                          int d, int bs, int max_blocks, int64_t num_blocks, int in_dtype,
+                          int pool_dtype, const float* k_scale, const float* v_scale,
+                          hipStream_t stream);
 int launch_split_reduce(const DecodeArgs& a);
 
 }  // namespace aicomp

@@ -401,8 +401,8 @@ constexpr int SK_MAX_SEQS = 1024;
 struct StreamKParams {
     void* out;
     const void* query;
-    const void* k_pool;
-    const void* v_pool;
+    void* k_pool;
+    void* v_pool;
     const int32_t* block_table;
     int64_t block_table_stride;
     const int32_t* context_lens;
@@ -414,7 +414,59 @@ struct StreamKParams {
     int num_waves;
     float* ws_acc;      // [slots][G][D]
     float* ws_ml;       // [slots][G][2]
+    // fused append (optional): row b of new_key / new_value is token context_lens[b]-1
+    const bf16_t* new_key;
+    const bf16_t* new_value;
+    int64_t new_token_stride, new_head_stride;     // elements
 };
+
+// 8 floats -> 8 e4m3 codes: clamp(x / scale, +-448), round to nearest even
+__device__ __forceinline__ uint2 quant8_fp8(const uint4& bf, float scale) {
+    const uint32_t w[4] = {bf.x, bf.y, bf.z, bf.w};
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = fminf(fmaxf(__uint_as_float(w[i] << 16) / scale, -448.f), 448.f);
+        f[2 * i + 1] = fminf(fmaxf(__uint_as_float(w[i] & 0xffff0000u) / scale, -448.f), 448.f);
+    }
+    int lo = 0, hi = 0;
+    lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], lo, false);
+    lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
+    hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], hi, false);
+    hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
+    return make_uint2((uint32_t)lo, (uint32_t)hi);
+}
+
+// Fused append: the row's last tile holds the sequence's newest token, whose K/V are not in
+// the pool yet.  The 16 lanes that own that row take it from new_key / new_value instead of
+// what they loaded, and write it to the pool (the append itself).  No other wave of this
+// launch reads that token, so no cross-wave ordering is needed.
+template <bool FP8>
+__device__ __forceinline__ void inject_new_row(TileRegs<FP8>& kr, TileRegs<FP8>& vr,
+                                               const StreamKParams& p, int seq, int kvh, int lane,
+                                               int tile_start, int len, int64_t b0, int64_t b1) {
+    const int tau = len - 1 - tile_start;              // 0..31, wave-uniform
+    const int c = lane & 15, q = lane >> 4;
+    const int64_t src = (int64_t)seq * p.new_token_stride + (int64_t)kvh * p.new_head_stride + 8 * c;
+    const uint4 nk = *(const uint4*)(p.new_key + src);
+    const uint4 nv = *(const uint4*)(p.new_value + src);
+    const bool mine = (tau & 3) == q;
+    const int64_t blk = tau < 16 ? b0 : b1;
+    const int64_t dst = ((blk * p.hkv + kvh) * BS + (tau & 15)) * (D / 8) + c;   // 8-element chunks
+    if constexpr (FP8) {
+        const uint2 ck = quant8_fp8(nk, p.k_scale[kvh]);
+        const uint2 cv = quant8_fp8(nv, p.v_scale[kvh]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (mine && i == (tau >> 2)) { kr.r[i] = ck; vr.r[i] = cv; }
+        if (mine) { ((uint2*)p.k_pool)[dst] = ck; ((uint2*)p.v_pool)[dst] = cv; }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (mine && i == (tau >> 2)) { kr.r[i] = nk; vr.r[i] = nv; }
+        if (mine) { ((uint4*)p.k_pool)[dst] = nk; ((uint4*)p.v_pool)[dst] = nv; }
+    }
+}
 
 __device__ __forceinline__ int sk_tiles(int len, int max_blocks) {
     len = min(max(len, 0), max_blocks * BS);
@@ -548,6 +600,10 @@ streamk_decode_kernel(StreamKParams p) {
                                            p.hkv, kvh, lane, g4, (t + k) * TILE, len, cmul);
         }
         const int tile_start = (t + k) * TILE;
+        if (p.new_key != nullptr && t + k == row_tiles - 1) {       // the row's newest token lives here
+            tile_blocks(k, b0, b1);
+            inject_new_row<FP8>(kr, vr, p, seq, kvh, lane, tile_start, len, b0, b1);
+        }
         if (tile_start + TILE > len)
             process_tile<FP8, false, true>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
                                            p.hkv, kvh, lane, g4, tile_start, len, cmul);
@@ -698,7 +754,7 @@ int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
     const int group = a.hq / a.hkv;
     const int64_t slots = SK_MAX_WAVES + a.rows * a.hkv;
     StreamKParams p;
-    p.out = a.out; p.query = a.query; p.k_pool = a.k_pool; p.v_pool = a.v_pool;
+    p.out = a.out; p.query = a.query; p.k_pool = (void*)a.k_pool; p.v_pool = (void*)a.v_pool;
     p.block_table = a.block_table; p.block_table_stride = a.block_table_stride;
     p.context_lens = a.context_lens;
     p.num_seqs = (int)a.rows; p.hq = a.hq; p.hkv = a.hkv; p.group = group; p.max_blocks = a.max_blocks;
@@ -708,6 +764,8 @@ int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
     p.num_waves = wgs * NWAVES;
     p.ws_acc = (float*)workspace;
     p.ws_ml = p.ws_acc + slots * group * D;
+    p.new_key = (const bf16_t*)a.new_key; p.new_value = (const bf16_t*)a.new_value;
+    p.new_token_stride = a.new_token_stride; p.new_head_stride = a.new_head_stride;
     if (a.kv_dtype == AICOMP_KV_FP8_E4M3)
         hipLaunchKernelGGL(streamk_decode_kernel<true>, dim3(wgs), dim3(256), 0, a.stream, p);
     else

@@ -95,6 +95,20 @@ class _PagedLayer:
         slots = self.slot_table[:, pos:pos + n].reshape(-1).contiguous()
         ops.kv_append(rows_k, rows_v, self.k_pool, self.v_pool, slots)
 
+    def decode_step(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, pos: int,
+                    group: int, scale: float) -> torch.Tensor:
+        """One decode step, append and attention in a single call: query ``[B, Hq, 1, D]``,
+        key/value ``[B, H, 1, D]`` written at position pos."""
+        B, Hq, _, D = query.shape
+        if key.shape[1] == self.kv_heads * group and group > 1:
+            key, value = key[:, ::group], value[:, ::group]
+        self.context_lens.fill_(pos + 1)
+        q = query[:, :, 0, :].contiguous()
+        out = torch.empty_like(q)
+        ops.paged_decode_attn(out, q, self.k_pool, self.v_pool, self.block_table, self.context_lens,
+                              scale, new_key=key[:, :, 0, :], new_value=value[:, :, 0, :])
+        return out.view(B, Hq, 1, D)
+
     def attend(self, query: torch.Tensor, pos: int, scale: float) -> torch.Tensor:
         """query ``[B, Hq, n, D]`` at positions pos..pos+n (rows already appended)."""
         B, Hq, n, D = query.shape
@@ -359,6 +373,9 @@ class CachedScaledDotProductAttention(nn.Module):
             if pos + n > self.max_seq_len:
                 raise RuntimeError(f"cache overflow: position {pos} + {n} new tokens > max_seq_len "
                                    f"{self.max_seq_len}")
+            if n == 1 and key.dtype == store.k_pool.dtype:
+                self.cache_pos = pos + 1          # decode step: append fused into the attention call
+                return store.decode_step(query, key, value, pos, self._group, scale)
             store.append(key, value, pos, self._group)
         self.cache_pos = pos + n
         # the caller's attn_mask is dropped, as in the reference (kv_cache.py:400-415): decode sees

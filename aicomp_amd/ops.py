@@ -118,11 +118,17 @@ def paged_decode_attn(out: torch.Tensor, query: torch.Tensor, k_pool: torch.Tens
                       context_lens: torch.Tensor, scale: float,
                       k_scale: Optional[torch.Tensor] = None,
                       v_scale: Optional[torch.Tensor] = None, partition_size: int = 0,
-                      workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      workspace: Optional[torch.Tensor] = None,
+                      new_key: Optional[torch.Tensor] = None,
+                      new_value: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``out[b, h] = softmax(q[b, h] . K_b^T * scale) V_b`` over the paged context.
 
     ``out``/``query`` ``[B, Hq, D]``; ``block_table [B, max_blocks]`` int32;
     ``context_lens [B]`` int32.  In place on ``out``, on the current stream.
+
+    With ``new_key`` / ``new_value`` ``[B, Hkv, D]`` the call first appends row b as token
+    ``context_lens[b] - 1`` of sequence b (the pools are written) - one decode step of the
+    reference operator in one call.
     """
     lib = _lib.load()
     _req(query.is_cuda, "tensors must live on a ROCm device (there is no CPU path)")
@@ -146,6 +152,22 @@ def paged_decode_attn(out: torch.Tensor, query: torch.Tensor, k_pool: torch.Tens
     if workspace is None:
         workspace = _workspace(query.device, need)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    if new_key is not None:
+        _req(new_value is not None and new_key.shape == (B, hkv, d) and new_value.shape == (B, hkv, d)
+             and new_key.dtype == query.dtype and new_value.dtype == query.dtype,
+             f"new_key/new_value must both be [{B}, {hkv}, {d}] of the query dtype")
+        _dev(new_key, query, "new_key")
+        _dev(new_value, query, "new_value")
+        if new_key.stride(2) != 1 or new_key.stride() != new_value.stride():
+            new_key, new_value = new_key.contiguous(), new_value.contiguous()
+        rc = lib.aicomp_paged_decode_attn_append(
+            out.data_ptr(), query.data_ptr(), new_key.data_ptr(), new_value.data_ptr(),
+            new_key.stride(0), new_key.stride(1), k_pool.data_ptr(), v_pool.data_ptr(),
+            block_table.data_ptr(), block_table.stride(0), context_lens.data_ptr(), B, hq, hkv, d, bs,
+            block_table.shape[1], nb, float(scale), qd, kd, _ptr(ks), _ptr(vs), partition_size,
+            _ptr(workspace), ws_bytes, _stream(query))
+        _lib.check(rc, lib)
+        return out
     rc = lib.aicomp_paged_decode_attn(out.data_ptr(), query.data_ptr(), k_pool.data_ptr(),
                                       v_pool.data_ptr(), block_table.data_ptr(),
                                       block_table.stride(0), context_lens.data_ptr(), B, hq, hkv, d,

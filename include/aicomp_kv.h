@@ -86,9 +86,10 @@ int aicomp_kv_append(const void* key, const void* value,
  *   kv_dtype FP8    k_scale / v_scale [Hkv] float dequantisation factors, fused
  *                   into the loads
  *   partition_size  split-K (flash-decoding) tokens per partition; 0 = choose
- *                   from the shape; a multiple of block_size otherwise.  With
- *                   more than one partition a second kernel merges the
- *                   partial (max, sum, output) triples.
+ *                   from the shape (balanced schedule: every wave gets the same
+ *                   number of 32-token tiles); a multiple of block_size otherwise.
+ *                   Split work is merged by a second kernel from partial
+ *                   (max, sum, output) triples.
  *   workspace       device scratch of at least
  *                   aicomp_paged_decode_workspace_bytes(...) bytes (may be NULL
  *                   when that returns 0), 16-byte aligned.  Its leading
@@ -110,6 +111,33 @@ int aicomp_paged_decode_attn(void* out, const void* query,
                              int partition_size,
                              void* workspace, size_t workspace_bytes,
                              void* stream);
+
+/*
+ * Append of one new token per sequence fused with decode attention: what one decode-step
+ * call of the reference operator does (kv_cache.py:383-403: store the new K/V row at the
+ * write position, then attend over the whole prefix), in a single main kernel.
+ *
+ *   new_key, new_value  [B, Hkv, D] of q_dtype, element (b,h,d) at
+ *                       b*kv_token_stride + h*kv_head_stride + d; row b becomes token
+ *                       context_lens[b] - 1 of sequence b (its slot comes from the block
+ *                       table), quantised with k_scale / v_scale for an fp8 pool
+ *   context_lens        lengths INCLUDING the new token
+ * Everything else as aicomp_paged_decode_attn.  The result equals aicomp_kv_append of those
+ * rows followed by aicomp_paged_decode_attn: the pool contents are bit-identical.
+ */
+int aicomp_paged_decode_attn_append(void* out, const void* query,
+                                    const void* new_key, const void* new_value,
+                                    int64_t kv_token_stride, int64_t kv_head_stride,
+                                    void* k_pool, void* v_pool,
+                                    const int32_t* block_table, int64_t block_table_stride,
+                                    const int32_t* context_lens,
+                                    int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                                    int block_size, int max_blocks_per_seq, int64_t num_blocks,
+                                    float scale, int q_dtype, int kv_dtype,
+                                    const float* k_scale, const float* v_scale,
+                                    int partition_size,
+                                    void* workspace, size_t workspace_bytes,
+                                    void* stream);
 
 size_t aicomp_paged_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads,
                                            int head_dim, int block_size,

@@ -194,3 +194,51 @@ def test_config3_long_context_split(device):
     got1 = to_f64(run_decode(w, w.block_table.shape[1] * 16))      # one partition
     assert_close_attn(got1, want, BF16_ATOL, BF16_RTOL, "unsplit")
     assert np.abs(got - got1).max() <= 2e-3
+
+
+@pytest.mark.parametrize("name,batch", [("llama3_8b_decode", 5), ("llama3_70b_decode_fp8", 3),
+                                        ("decode_fp32_small", 4)])
+def test_fused_append_decode_equals_append_then_decode(device, name, batch):
+    """One call that appends the new token and attends == kv_append followed by decode:
+    pools bit-identical, outputs bit-identical (same kernel, same values)."""
+    w = workloads.make_workload("x", device=device, seed=7, shape=small(name, batch=batch))
+    k2, v2 = w.k_pool.clone(), w.v_pool.clone()
+    ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping, w.k_scale, w.v_scale)
+    ref = run_decode(w)
+    out = torch.full_like(w.query, float("nan"))
+    ops.paged_decode_attn(out, w.query, k2, v2, w.block_table, w.context_lens, w.scale,
+                          k_scale=w.k_scale, v_scale=w.v_scale, new_key=w.new_key, new_value=w.new_value)
+    torch.cuda.synchronize()
+    bits = lambda t: t.view(torch.uint8) if t.dtype == torch.float8_e4m3fn else t
+    assert torch.equal(bits(k2), bits(w.k_pool)) and torch.equal(bits(v2), bits(w.v_pool))
+    assert torch.equal(out.view(torch.int16 if out.dtype == torch.bfloat16 else torch.int32),
+                       ref.view(torch.int16 if ref.dtype == torch.bfloat16 else torch.int32))
+    # explicit partition size: the append runs as its own kernel in front of the grid kernel
+    k3, v3 = k2.clone(), v2.clone()
+    k3.view(torch.uint8).zero_()
+    ops.paged_decode_attn(out, w.query, k2, v2, w.block_table, w.context_lens, w.scale,
+                          k_scale=w.k_scale, v_scale=w.v_scale, new_key=w.new_key, new_value=w.new_value,
+                          partition_size=256)
+    assert torch.equal(bits(k2), bits(w.k_pool))
+    assert_close_attn(to_f64(out), to_f64(ref), 2e-3, 0.0, "fused, grid schedule")
+
+
+def test_fused_append_edge_positions(device):
+    """New token at a tile start, tile end, block start, and as the very first token."""
+    sh = workloads.Shape("t", 6, 8, 2, 128, ctx_lo=100, ctx_hi=100)
+    w = workloads.make_workload("t", device=device, seed=9, shape=sh)
+    ctx = torch.tensor([1, 32, 33, 64, 49, 100], dtype=torch.int32, device=device)
+    k2, v2 = w.k_pool.clone(), w.v_pool.clone()
+    bs = 16
+    pos = (ctx - 1).long()
+    slots = w.block_table[torch.arange(6, device=device), pos // bs].long() * bs + pos % bs
+    ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, slots)
+    ref = run_decode(w, ctx=ctx)
+    out = torch.empty_like(w.query)
+    ops.paged_decode_attn(out, w.query, k2, v2, w.block_table, ctx, w.scale, new_key=w.new_key,
+                          new_value=w.new_value)
+    assert torch.equal(k2.view(torch.int16), w.k_pool.view(torch.int16))
+    assert torch.equal(v2.view(torch.int16), w.v_pool.view(torch.int16))
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+    want = oracle_decode(w, ctx=ctx.cpu().numpy())
+    assert_close_attn(to_f64(out), want, BF16_ATOL, BF16_RTOL, "fused edge positions")
