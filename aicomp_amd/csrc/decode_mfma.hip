@@ -147,17 +147,17 @@ template <bool FP8, bool NEXT, bool MASK>
 __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, TileRegs<FP8>& vr,
                                              const bf16x8_t (&qf)[4], unsigned char* kt, int wr_off,
                                              int rd_off, const void* k_pool, const void* v_pool,
-                                             int64_t nb0, int64_t nb1, int hkv, int kvh, int lane,
+                                             int64_t nb0, int64_t nb1, int hkv, int kvh_next, int lane,
                                              int g4, int tile_start, int end, float cmul) {
 #ifdef EXP_LOADS_ONLY
     {
         uint4 x = make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < 8; ++i) { uint4 a = tile_bf16<FP8>(kr, i); x.x ^= a.x; x.y ^= a.y; x.z ^= a.z; x.w ^= a.w; }
-        if (NEXT) load_tile<FP8>(kr, k_pool, nb0, nb1, hkv, kvh, lane);
+        if (NEXT) load_tile<FP8>(kr, k_pool, nb0, nb1, hkv, kvh_next, lane);
 #pragma unroll
         for (int i = 0; i < 8; ++i) { uint4 a = tile_bf16<FP8>(vr, i); x.x ^= a.x; x.y ^= a.y; x.z ^= a.z; x.w ^= a.w; }
-        if (NEXT) load_tile<FP8>(vr, v_pool, nb0, nb1, hkv, kvh, lane);
+        if (NEXT) load_tile<FP8>(vr, v_pool, nb0, nb1, hkv, kvh_next, lane);
         st.O[0][0] += __uint_as_float(x.x ^ x.y ^ x.z ^ x.w);
         return;
     }
@@ -166,7 +166,7 @@ __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, T
 #pragma unroll
     for (int i = 0; i < 8; ++i)
         *(uint4*)(kt + wr_off + i * 4 * KROW) = tile_bf16<FP8>(kr, i);
-    if (NEXT) load_tile<FP8>(kr, k_pool, nb0, nb1, hkv, kvh, lane);
+    if (NEXT) load_tile<FP8>(kr, k_pool, nb0, nb1, hkv, kvh_next, lane);
 
     // ---- S^T = K Q^T for the two 16-token sub-tiles
     f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
@@ -230,7 +230,7 @@ __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, T
         af[j].z = __builtin_amdgcn_perm(v0[4 * 5 + (j >> 1)], v0[4 * 4 + (j >> 1)], sel);
         af[j].w = __builtin_amdgcn_perm(v0[4 * 7 + (j >> 1)], v0[4 * 6 + (j >> 1)], sel);
     }
-    if (NEXT) load_tile<FP8>(vr, v_pool, nb0, nb1, hkv, kvh, lane);
+    if (NEXT) load_tile<FP8>(vr, v_pool, nb0, nb1, hkv, kvh_next, lane);
 #pragma unroll
     for (int j = 0; j < 8; ++j)
         st.O[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, af[j]), pf, st.O[j], 0, 0, 0);
@@ -414,6 +414,7 @@ struct StreamKParams {
     int num_waves;
     float* ws_acc;      // [slots][G][D]
     float* ws_ml;       // [slots][G][2]
+    int* ws_rows;       // [rows][2]: first and last wave holding a partial of the row
     // fused append (optional): row b of new_key / new_value is token context_lens[b]-1
     const bf16_t* new_key;
     const bf16_t* new_value;
@@ -479,7 +480,7 @@ __device__ __forceinline__ int sk_wave_of(int64_t g, int64_t N, int W) {
 }
 
 template <bool FP8>
-__global__ void __launch_bounds__(256, 2)
+__global__ void __launch_bounds__(256, 1)     // one workgroup per CU: a wave may use the whole register file
 streamk_decode_kernel(StreamKParams p) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -492,9 +493,22 @@ streamk_decode_kernel(StreamKParams p) {
     __shared__ int wave_tot[NWAVES];
     unsigned char* kt = lds + w * KTILE_BYTES;
 
-    // ---- prologue: tiles per sequence -> exclusive prefix sums (4 sequences per thread)
-    {
-        int loc[4], sum = 0;
+    // ---- prologue: tiles per sequence -> exclusive prefix sums
+    if (B <= 64) {
+        // every wave scans for itself and reads back only what it wrote: no barrier (the
+        // four waves write identical values to the same words)
+        const int mine = lane < B ? sk_tiles(p.context_lens[lane], p.max_blocks) : 0;
+        int inc = mine;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int v = __shfl_up(inc, o);
+            if (lane >= o) inc += v;
+        }
+        prefix[lane] = inc - mine;
+        if (lane == 63) prefix[64] = inc;
+        if (B < 64 && lane == B) prefix[B] = inc - mine;      // == total: lanes >= B add nothing
+    } else {
+        int loc[4], sum = 0;                                  // 4 sequences per thread
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const int sidx = 4 * tid + k;
@@ -550,26 +564,48 @@ streamk_decode_kernel(StreamKParams p) {
     const int wr_off = (lane >> 4) * KROW + (lane & 15) * 16;
     const int rd_off = (4 * (r16 & 3) + (r16 >> 2)) * KROW + g4 * 16;
 
-    for (int64_t g = g0; g < g1 && seq < B;) {
-        const int nt = (int)min((int64_t)(row_tiles - t), g1 - g);       // tiles of this segment (>= 1)
-        const int len = min(p.context_lens[seq], p.max_blocks * BS);
-
-        // Q rows and the table slice of the segment, one wait for both
-        const int32_t* table = p.block_table + (int64_t)seq * p.block_table_stride;
-        const int blk_base = 2 * t;
-        int tab_first = 0;
-        int tab = (blk_base + lane < p.max_blocks) ? table[blk_base + lane] : 0;
-        bf16x8_t qf[4];
-        {
-            const uint4* qp = (const uint4*)((const bf16_t*)p.query +
-                                             ((int64_t)seq * p.hq + kvh * G + min(r16, G - 1)) * D + 8 * g4);
+    // ---- segments.  A segment is the part of one (sequence, KV head) row that falls into this
+    // wave's tile range.  The next segment's query rows and table slice are requested while the
+    // current one streams, and its first K/V tile is prefetched by the current segment's last
+    // tile, so the loads never drain at a row boundary.
+    // raw query rows of (sequence, KV head); columns beyond the group are zeroed by q_operand
+    // only when the rows are used, so that issuing the loads never waits for them
+    auto load_q = [&](int sq, int kh, uint4 (&q)[4]) {
+        const uint4* qp = (const uint4*)((const bf16_t*)p.query +
+                                         ((int64_t)sq * p.hq + kh * G + min(r16, G - 1)) * D + 8 * g4);
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                uint4 v = qp[s * 4];
-                if (r16 >= G) v = make_uint4(0, 0, 0, 0);
-                qf[s] = __builtin_bit_cast(bf16x8_t, v);
-            }
-        }
+        for (int s = 0; s < 4; ++s) q[s] = qp[s * 4];
+    };
+    auto q_operand = [&](const uint4 (&raw)[4], bf16x8_t (&q)[4]) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+            q[s] = __builtin_bit_cast(bf16x8_t, r16 < G ? raw[s] : make_uint4(0, 0, 0, 0));
+    };
+    auto load_tab = [&](int sq, int first_block) {
+        const int32_t* table = p.block_table + (int64_t)sq * p.block_table_stride;
+        return (first_block + lane < p.max_blocks) ? table[first_block + lane] : 0;
+    };
+
+    int nt = (int)min((int64_t)(row_tiles - t), g1 - g0);          // tiles of the current segment (>= 1)
+    bf16x8_t qf[4];
+    uint4 qraw[4];
+    load_q(seq, kvh, qraw);
+    int tab = load_tab(seq, 2 * t);
+    TileRegs<FP8> kr, vr;
+    {
+        __builtin_amdgcn_s_waitcnt(0x0F70);                        // Q and table have landed
+        q_operand(qraw, qf);
+        const int64_t b0 = clamp_block(__builtin_amdgcn_readlane(tab, 0), p.num_blocks);
+        const int64_t b1 = clamp_block(__builtin_amdgcn_readlane(tab, 1), p.num_blocks);
+        load_tile<FP8>(kr, p.k_pool, b0, b1, p.hkv, kvh, lane);
+        load_tile<FP8>(vr, p.v_pool, b0, b1, p.hkv, kvh, lane);
+    }
+
+    for (int64_t g = g0; g < g1 && seq < B;) {
+        const int len = min(p.context_lens[seq], p.max_blocks * BS);
+        const int blk_base = 2 * t;
+        const int32_t* table = p.block_table + (int64_t)seq * p.block_table_stride;
+        int tab_first = 0;
         const float cmul = p.qk_mul * (FP8 ? p.k_scale[kvh] : 1.f);
         auto tile_blocks = [&](int k, int64_t& b0, int64_t& b1) {      // k-th tile of the segment
             const int i0 = 2 * k;
@@ -582,17 +618,28 @@ streamk_decode_kernel(StreamKParams p) {
             b1 = clamp_block(__builtin_amdgcn_readlane(tab, i0 + 1 - tab_first), p.num_blocks);
         };
 
+        // the segment after this one (same wave): next KV head, or the next sequence with tokens
+        int nseq = seq, nkvh = kvh + 1, nrow_tiles = row_tiles;
+        const bool more = g + nt < g1;
+        if (more && nkvh == p.hkv) {
+            nkvh = 0;
+            do { ++nseq; } while (nseq < B && __builtin_amdgcn_readfirstlane(prefix[nseq + 1] - prefix[nseq]) == 0);
+            nrow_tiles = nseq < B ? __builtin_amdgcn_readfirstlane(prefix[nseq + 1] - prefix[nseq]) : 0;
+        }
+        const bool has_next = more && nseq < B;
+        int tabn = 0;
+        bf16x8_t qn[4];
+        if (has_next) {
+            load_q(nseq, nkvh, qraw);
+            tabn = load_tab(nseq, 0);
+        }
+
         WaveState st;
         st.m = NEG_BIG; st.lsum = 0.f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) st.O[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-        TileRegs<FP8> kr, vr;
         int64_t b0, b1;
-        __builtin_amdgcn_s_waitcnt(0x0F70);          // Q and table have landed
-        tile_blocks(0, b0, b1);
-        load_tile<FP8>(kr, p.k_pool, b0, b1, p.hkv, kvh, lane);
-        load_tile<FP8>(vr, p.v_pool, b0, b1, p.hkv, kvh, lane);
         int k = 0;
         for (; k + 1 < nt; ++k) {
             tile_blocks(k + 1, b0, b1);
@@ -604,12 +651,22 @@ streamk_decode_kernel(StreamKParams p) {
             tile_blocks(k, b0, b1);
             inject_new_row<FP8>(kr, vr, p, seq, kvh, lane, tile_start, len, b0, b1);
         }
-        if (tile_start + TILE > len)
+        // The segment's last tile always runs the masked body (a full tile simply masks nothing):
+        // one prefetching call site, so the prefetched registers need no merging afterwards.
+        int tab_ready = 0;
+        if (has_next) {
+            // prefetch the first tile of the next segment
+            __builtin_amdgcn_s_waitcnt(0x0F70);      // next Q rows and table slice (and this tile) have landed
+            q_operand(qraw, qn);
+            tab_ready = tabn;
+            b0 = clamp_block(__builtin_amdgcn_readlane(tab_ready, 0), p.num_blocks);
+            b1 = clamp_block(__builtin_amdgcn_readlane(tab_ready, 1), p.num_blocks);
+            process_tile<FP8, true, true>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, b0, b1,
+                                          p.hkv, nkvh, lane, g4, tile_start, len, cmul);
+        } else {
             process_tile<FP8, false, true>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
                                            p.hkv, kvh, lane, g4, tile_start, len, cmul);
-        else
-            process_tile<FP8, false, false>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
-                                            p.hkv, kvh, lane, g4, tile_start, len, cmul);
+        }
 
         // ---- flush: lane (head r16, g4) holds O^T[dim 32*g4 + 8*i + j][head] in O[j][i]
         float lsum = st.lsum;
@@ -625,95 +682,73 @@ streamk_decode_kernel(StreamKParams p) {
             }
             if (g4 == 0) *(float2*)(p.ws_ml + (slot * G + r16) * 2) = make_float2(st.m, lsum);
         }
-
-        // ---- next row
-        g += nt;
-        t = 0;
-        if (++kvh == p.hkv) {
-            kvh = 0;
-            do { ++seq; } while (seq < B && __builtin_amdgcn_readfirstlane(prefix[seq + 1] - prefix[seq]) == 0);
-            if (seq < B) row_tiles = __builtin_amdgcn_readfirstlane(prefix[seq + 1] - prefix[seq]);
+        // the waves holding a row's first and last tile tell the merge kernel where its partials are
+        if (lane == 0) {
+            int* rm = p.ws_rows + 2 * ((int64_t)seq * p.hkv + kvh);
+            if (t == 0) rm[0] = wave_id;
+            if (t + nt == row_tiles) rm[1] = wave_id;
         }
+
+        // ---- next segment
+        g += nt;
+        if (!has_next) break;
+        seq = nseq; kvh = nkvh; row_tiles = nrow_tiles; t = 0;
+        nt = (int)min((int64_t)row_tiles, g1 - g);
+        tab = tab_ready;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) qf[s] = qn[s];
     }
 }
 
-// Merge of the balanced schedule's partials: one workgroup per (KV head, sequence, head of
-// the group).  The row's partials sit in consecutive slots first+row .. last+row; their
-// weights 2^(m_i - M) are computed once (one lane per partial) and parked in LDS, then each
-// lane accumulates one output dim with independent loads.
-constexpr int SK_RED_CACHE = 512;
-
-__global__ void __launch_bounds__(128)
+// Merge of the balanced schedule's partials: one wave per (KV head, sequence, head of the
+// group).  The row's partials sit in consecutive slots first+row .. last+row (first / last
+// wave recorded by the main kernel); their weights 2^(m_i - M) are computed once (one lane
+// per partial) and parked in LDS, then each lane accumulates two output dims with
+// independent loads.  A single wave: reductions are shuffles, no barrier.
+__global__ void __launch_bounds__(64)
 streamk_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws_acc,
-                      const float* __restrict__ ws_ml, const int32_t* __restrict__ context_lens,
-                      int num_seqs, int hq, int hkv, int group, int max_blocks, int num_waves,
+                      const float* __restrict__ ws_ml, const int* __restrict__ ws_rows,
+                      const int32_t* __restrict__ context_lens, int hq, int hkv, int group,
                       const float* __restrict__ v_scale) {
     const int kvh = blockIdx.x, seq = blockIdx.y, h = blockIdx.z;
-    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    __shared__ int redi[2][2];
-    __shared__ float redf[2][2];
-    __shared__ float wgt[SK_RED_CACHE];
-    // tiles before this sequence, and in total
-    int before = 0, total = 0;
-    for (int sidx = tid; sidx < num_seqs; sidx += 128) {
-        const int tl = sk_tiles(context_lens[sidx], max_blocks);
-        total += tl;
-        if (sidx < seq) before += tl;
-    }
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) { before += __shfl_xor(before, o); total += __shfl_xor(total, o); }
-    if (lane == 0) { redi[0][wv] = before; redi[1][wv] = total; }
-    __syncthreads();
-    before = redi[0][0] + redi[0][1];
-    total = redi[1][0] + redi[1][1];
-    const int row_tiles = sk_tiles(context_lens[seq], max_blocks);
+    const int lane = threadIdx.x;
+    __shared__ float wgt[SK_MAX_WAVES / 4];
+    const int64_t row = (int64_t)seq * hkv + kvh;
     bf16_t* o = out + ((int64_t)seq * hq + kvh * group + h) * D;
-    if (row_tiles == 0) {
-        o[tid].bits = 0;
+    if (context_lens[seq] <= 0) {            // no tiles, no partials: the output row is zero
+        o[lane].bits = 0; o[lane + 64].bits = 0;
         return;
     }
-    const int64_t N = (int64_t)hkv * total;
-    const int W = (int)min((int64_t)num_waves, N);        // every one of the W waves owns >= 1 tile
-    const int64_t gr = (int64_t)hkv * before + (int64_t)kvh * row_tiles;
-    const int first = sk_wave_of(gr, N, W);
-    const int last = sk_wave_of(gr + row_tiles - 1, N, W);
+    const int first = ws_rows[2 * row], last = ws_rows[2 * row + 1];
     const int np = last - first + 1;
-    const int64_t row = (int64_t)seq * hkv + kvh;
     const float* ml = ws_ml + ((first + row) * group + h) * 2;          // partial i at ml[i * group * 2]
-    const float* acc = ws_acc + ((first + row) * group + h) * D + tid;  // partial i at acc[i * group * D]
+    const float* acc = ws_acc + ((first + row) * group + h) * D + lane; // partial i at acc[i * group * D]
     float mx = NEG_BIG;
-    for (int i = tid; i < np; i += 128) mx = fmaxf(mx, ml[(int64_t)i * group * 2]);
+    for (int i = lane; i < np; i += 64) mx = fmaxf(mx, ml[(int64_t)i * group * 2]);
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-    if (lane == 0) redf[0][wv] = mx;
-    __syncthreads();
-    mx = fmaxf(redf[0][0], redf[0][1]);
     float den = 0.f;
-    for (int i = tid; i < np; i += 128) {
-        const float f = exp2f(ml[(int64_t)i * group * 2] - mx);
-        if (i < SK_RED_CACHE) wgt[i] = f;
-        den = fmaf(f, ml[(int64_t)i * group * 2 + 1], den);
+    for (int i = lane; i < np; i += 64) {
+        const float2 v = *(const float2*)(ml + (int64_t)i * group * 2);
+        const float f = exp2f(v.x - mx);
+        wgt[i] = f;
+        den = fmaf(f, v.y, den);
     }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) den += __shfl_xor(den, off);
-    if (lane == 0) redf[1][wv] = den;
-    __syncthreads();
-    den = redf[1][0] + redf[1][1];
     const int64_t stride = (int64_t)group * D;
-    float num = 0.f;
+    float n0 = 0.f, n1 = 0.f;
     int i = 0;
-    for (; i + 4 <= np && i + 4 <= SK_RED_CACHE; i += 4) {
-        const float a0 = acc[i * stride], a1 = acc[(i + 1) * stride];
-        const float a2 = acc[(i + 2) * stride], a3 = acc[(i + 3) * stride];
-        num = fmaf(wgt[i], a0, num); num = fmaf(wgt[i + 1], a1, num);
-        num = fmaf(wgt[i + 2], a2, num); num = fmaf(wgt[i + 3], a3, num);
+    for (; i + 2 <= np; i += 2) {
+        const float a0 = acc[i * stride], b0 = acc[i * stride + 64];
+        const float a1 = acc[(i + 1) * stride], b1 = acc[(i + 1) * stride + 64];
+        n0 = fmaf(wgt[i], a0, n0); n1 = fmaf(wgt[i], b0, n1);
+        n0 = fmaf(wgt[i + 1], a1, n0); n1 = fmaf(wgt[i + 1], b1, n1);
     }
-    for (; i < np; ++i) {
-        const float f = i < SK_RED_CACHE ? wgt[i] : exp2f(ml[(int64_t)i * group * 2] - mx);
-        num = fmaf(f, acc[i * stride], num);
-    }
-    const float vs = v_scale ? v_scale[kvh] : 1.f;
-    o[tid].bits = f32_to_bf16(den > 0.f ? vs * num / den : 0.f);
+    if (i < np) { n0 = fmaf(wgt[i], acc[i * stride], n0); n1 = fmaf(wgt[i], acc[i * stride + 64], n1); }
+    const float inv = den > 0.f ? (v_scale ? v_scale[kvh] : 1.f) / den : 0.f;
+    o[lane].bits = f32_to_bf16(n0 * inv);
+    o[lane + 64].bits = f32_to_bf16(n1 * inv);
 }
 
 }  // namespace
@@ -733,7 +768,7 @@ bool decode_streamk_supported(const DecodeArgs& a) {
 
 size_t decode_streamk_workspace_bytes(int64_t rows, int hq, int hkv, int d) {
     const int64_t slots = SK_MAX_WAVES + rows * hkv;
-    return (size_t)slots * (hq / hkv) * (size_t)(d + 2) * sizeof(float);
+    return (size_t)slots * (hq / hkv) * (size_t)(d + 2) * sizeof(float) + (size_t)rows * hkv * 2 * sizeof(int);
 }
 
 int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
@@ -764,6 +799,7 @@ int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
     p.num_waves = wgs * NWAVES;
     p.ws_acc = (float*)workspace;
     p.ws_ml = p.ws_acc + slots * group * D;
+    p.ws_rows = (int*)(p.ws_ml + slots * group * 2);
     p.new_key = (const bf16_t*)a.new_key; p.new_value = (const bf16_t*)a.new_value;
     p.new_token_stride = a.new_token_stride; p.new_head_stride = a.new_head_stride;
     if (a.kv_dtype == AICOMP_KV_FP8_E4M3)
@@ -771,9 +807,9 @@ int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
     else
         hipLaunchKernelGGL(streamk_decode_kernel<false>, dim3(wgs), dim3(256), 0, a.stream, p);
     AICOMP_HIP_LAUNCH_CHECK();
-    hipLaunchKernelGGL(streamk_reduce_kernel, dim3(a.hkv, (unsigned)a.rows, group), dim3(128), 0, a.stream,
-                       (bf16_t*)a.out, p.ws_acc, p.ws_ml, a.context_lens, (int)a.rows, a.hq, a.hkv, group,
-                       a.max_blocks, p.num_waves, a.v_scale);
+    hipLaunchKernelGGL(streamk_reduce_kernel, dim3(a.hkv, (unsigned)a.rows, group), dim3(64), 0, a.stream,
+                       (bf16_t*)a.out, p.ws_acc, p.ws_ml, p.ws_rows, a.context_lens, a.hq, a.hkv, group,
+                       a.v_scale);
     AICOMP_HIP_LAUNCH_CHECK();
     return AICOMP_KV_OK;
 }
