@@ -20,25 +20,37 @@
 
 namespace aicomp {
 
+// K/V rows are read once per call: non-temporal loads (streaming, no reuse in L2)
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 stream_ld16(const void* p) {
+    u32x4_t v = __builtin_nontemporal_load((const u32x4_t*)p);
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ uint2 stream_ld8(const void* p) {
+    u32x2_t v = __builtin_nontemporal_load((const u32x2_t*)p);
+    return make_uint2(v[0], v[1]);
+}
+
 template <typename KV_T> struct KvLoad;
 template <> struct KvLoad<float> {
     static constexpr int N = 4;
     __device__ __forceinline__ static void load(const float* p, float* f) {
-        uint4 r = *reinterpret_cast<const uint4*>(p);
+        uint4 r = stream_ld16(p);
         Vec16<float>::unpack(r, f);
     }
 };
 template <> struct KvLoad<bf16_t> {
     static constexpr int N = 8;
     __device__ __forceinline__ static void load(const bf16_t* p, float* f) {
-        uint4 r = *reinterpret_cast<const uint4*>(p);
+        uint4 r = stream_ld16(p);
         Vec16<bf16_t>::unpack(r, f);
     }
 };
 template <> struct KvLoad<fp8_t> {
     static constexpr int N = 8;
     __device__ __forceinline__ static void load(const fp8_t* p, float* f) {
-        uint2 r = *reinterpret_cast<const uint2*>(p);
+        uint2 r = stream_ld8(p);
         const uint32_t w[2] = {r.x, r.y};
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
