@@ -27,7 +27,7 @@ METRIC = "decode-attn HBM GB/s (% peak) + tokens/s, Llama-3-8B paged KV, 1 GPU"
 
 # HBM bytes per decode launch of the Llama-3-8B shape from rocprofv3 --pmc
 # (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, the factors a 1 GiB device copy gives), main + merge kernel.
-MEASURED_TRAFFIC_BYTES = 651.9e6   # profiles/decode_llama3_8b_decode.md
+MEASURED_TRAFFIC_BYTES = 651.3e6   # profiles/decode_llama3_8b_decode.md
 
 
 def _events(n):
