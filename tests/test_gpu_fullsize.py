@@ -1,0 +1,111 @@
+"""The five benchmark shapes at their full sizes: properties that do not depend on the size
+(schedule agreement, fused == unfused, bit-exact scatter) plus the float64 oracle on a sample
+of sequences (the oracle walks tokens in Python, so a sample keeps the suite fast)."""
+import numpy as np
+import pytest
+import torch
+
+from aicomp_amd import ops, workloads
+from oracle import paged_kv_oracle as orc
+from helpers import NAME, assert_close_attn, raw, to_f64
+
+pytestmark = pytest.mark.gpu
+BF16_ATOL, BF16_RTOL = 1e-2, 2e-2
+
+
+def oracle_rows(w, rows, q, bt, ctx):
+    ks = None if w.k_scale is None else w.k_scale.cpu().numpy()
+    vs = None if w.v_scale is None else w.v_scale.cpu().numpy()
+    kp, vp = raw(w.k_pool), raw(w.v_pool)
+    idx = torch.tensor(rows)
+    return orc.paged_decode_attn(raw(q[idx.to(q.device)]), kp, vp, bt.cpu().numpy()[rows],
+                                 [int(ctx[r]) for r in rows], w.scale, NAME[q.dtype], NAME[w.k_pool.dtype],
+                                 ks, vs)
+
+
+def decode(w, q, bt, ctx, ps=0, **kw):
+    out = torch.full_like(q, float("nan"))
+    ops.paged_decode_attn(out, q, w.k_pool, w.v_pool, bt, ctx, w.scale, w.k_scale, w.v_scale,
+                          partition_size=ps, **kw)
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("name,sample", [("llama3_8b_decode", [0, 7, 31, 63]),
+                                         ("long_context_skewed", None),
+                                         ("llama3_70b_decode_fp8", [0, 64, 127])])
+def test_full_decode_shapes(device, name, sample):
+    w = workloads.make_workload(name, device=device)
+    k0, v0 = w.k_pool.clone(), w.v_pool.clone()
+    # fused append + decode (balanced schedule) on a copy of the pools
+    fused = torch.full_like(w.query, float("nan"))
+    ops.paged_decode_attn(fused, w.query, k0, v0, w.block_table, w.context_lens, w.scale, w.k_scale,
+                          w.v_scale, new_key=w.new_key, new_value=w.new_value)
+    # append, then decode
+    ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping, w.k_scale, w.v_scale)
+    bits = lambda t: t.view(torch.uint8) if t.dtype == torch.float8_e4m3fn else t.view(torch.int16)
+    assert torch.equal(bits(k0), bits(w.k_pool)) and torch.equal(bits(v0), bits(w.v_pool))
+    balanced = decode(w, w.query, w.block_table, w.context_lens)
+    assert torch.equal(fused.view(torch.int16), balanced.view(torch.int16))
+    grid = decode(w, w.query, w.block_table, w.context_lens, ps=1024)
+    assert (grid.float() - balanced.float()).abs().max() <= 2e-3
+    assert torch.isfinite(balanced.float()).all()
+    if sample is None:                                          # the two longest and the shortest
+        order = sorted(range(w.num_seqs), key=lambda i: w.ctx_list[i])
+        sample = [order[0], order[-2], order[-1]]
+    want = oracle_rows(w, sample, w.query, w.block_table, w.ctx_list)
+    got = to_f64(balanced)[sample]
+    assert_close_attn(got, want, BF16_ATOL, BF16_RTOL, f"{name} rows {sample}")
+
+
+def test_full_long_context_unsplit_equals_split(device):
+    w = workloads.make_workload("long_context_skewed", device=device)
+    ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping)
+    split = decode(w, w.query, w.block_table, w.context_lens)
+    whole = w.block_table.shape[1] * 16
+    unsplit = decode(w, w.query, w.block_table, w.context_lens, ps=(whole + 31) // 32 * 32)
+    assert (split.float() - unsplit.float()).abs().max() <= 2e-3
+    assert max(w.ctx_list) > 16384 and min(w.ctx_list) < 1024       # the batch really is skewed
+
+
+def test_full_chunked_prefill_mixed(device):
+    """All 2108 new rows scattered bit-exact, then prefill of the 4 chunks and decode of the 60."""
+    w = workloads.make_workload("chunked_prefill_mixed", device=device)
+    before_k, before_v = w.k_pool.clone(), w.v_pool.clone()
+    ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping)
+    sm, bs = w.slot_mapping, 16
+    assert sm.numel() == 2108 and sm.unique().numel() == 2108
+    before_k[sm // bs, :, sm % bs, :] = w.new_key
+    before_v[sm // bs, :, sm % bs, :] = w.new_value
+    assert torch.equal(before_k.view(torch.int16), w.k_pool.view(torch.int16))
+    assert torch.equal(before_v.view(torch.int16), w.v_pool.view(torch.int16))
+    npre = w.num_prefill_seqs
+    T = int(w.cu_q_lens[npre])
+    out = torch.full((T, 32, 128), float("nan"), dtype=torch.bfloat16, device=device)
+    ops.paged_prefill_attn(out, w.query[:T].contiguous(), w.k_pool, w.v_pool,
+                           w.block_table[:npre].contiguous(), w.context_lens[:npre].contiguous(),
+                           w.cu_q_lens[:npre + 1].contiguous(), w.scale, max_q_len=512)
+    dec = decode(w, w.query[T:].contiguous(), w.block_table[npre:].contiguous(),
+                 w.context_lens[npre:].contiguous())
+    assert torch.isfinite(out.float()).all() and torch.isfinite(dec.float()).all()
+    # last row of every chunk == decode of that row over the same context
+    last = [int(w.cu_q_lens[s + 1]) - 1 for s in range(npre)]
+    qd = w.query[last].contiguous()
+    d2 = decode(w, qd, w.block_table[:npre].contiguous(), w.context_lens[:npre].contiguous())
+    assert (d2.float() - out[last].float()).abs().max() <= 4e-3
+    want = oracle_rows(w, [npre, npre + 59], w.query[T - npre:], w.block_table, w.ctx_list)
+    # (rows npre.. of the decode part: index into the decode queries)
+    got = to_f64(dec)[[0, 59]]
+    assert_close_attn(got, want, BF16_ATOL, BF16_RTOL, "decode tail of the mixed step")
+
+
+def test_full_fp32_anchor_vs_cpu_reference_path(device):
+    """Config 1 against the reference's own CPU procedure (gather -> repeat_kv -> contiguous ->
+    torch SDPA, fp32), <= 1e-5."""
+    from oracle import contiguous_ref as cref
+    w = workloads.make_workload("decode_fp32_small", device=device)
+    ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping)
+    got = decode(w, w.query, w.block_table, w.context_lens)
+    want = cref.reference_cpu_decode(w.query.cpu(), w.k_pool.cpu(), w.v_pool.cpu(), w.block_table.cpu(),
+                                     w.context_lens.cpu(), w.scale)
+    assert (got.cpu() - want).abs().max().item() <= 1e-5
