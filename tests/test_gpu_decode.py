@@ -275,3 +275,26 @@ def test_fp8_all_codes_through_the_decode_kernel(device):
     got = out[:, 0, 0].float().cpu()
     assert torch.equal(got, want) or torch.equal(got.abs() + 0.0, want.abs() + 0.0) and \
         torch.equal(torch.signbit(got) | (got == 0), torch.signbit(want) | (want == 0))
+
+
+@pytest.mark.parametrize("batch", [65, 1024, 1030])
+def test_decode_many_short_sequences(device, batch):
+    """Large batches of short sequences: prefix sums over more than one wave, the 1024-sequence
+    limit of the balanced schedule, and the grid schedule beyond it."""
+    sh = workloads.Shape("t", batch, 8, 2, 128, ctx_lo=0, ctx_hi=90, kv_std=0.5)
+    w = workloads.make_workload("t", device=device, seed=11, shape=sh)
+    ctx = (w.context_lens - 1).clamp(min=0)                    # includes empty sequences
+    got = to_f64(run_decode(w, 0, ctx=ctx))
+    want = oracle_decode(w, ctx=ctx.cpu().numpy())
+    assert_close_attn(got, want, BF16_ATOL, BF16_RTOL, f"batch {batch}")
+    empty = (ctx == 0).cpu().numpy()
+    assert empty.any() and np.array_equal(got[empty], np.zeros_like(got[empty]))
+
+
+def test_decode_all_sequences_empty(device):
+    sh = workloads.Shape("t", 5, 8, 2, 128, ctx_lo=10, ctx_hi=20)
+    w = workloads.make_workload("t", device=device, shape=sh)
+    ctx = torch.zeros(5, dtype=torch.int32, device=device)
+    for ps in (0, 64):
+        out = run_decode(w, ps, ctx=ctx)
+        assert float(out.float().abs().sum()) == 0.0
