@@ -22,11 +22,14 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
+# Per-source extras.  The prefill kernel's row maxima read MFMA results directly; without this
+# flag every fmaxf operand is first canonicalised by a self-max (one extra VALU op per score).
+EXTRA_FLAGS = {"prefill_mfma.hip": ["-fno-honor-nans"]}
 
 
 def _compile(src: str) -> str:
     obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-    cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC, *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")

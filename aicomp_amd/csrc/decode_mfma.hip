@@ -38,7 +38,6 @@
 //              last partition (device-scope counter) merges them in the same
 //              launch, so a decode call is one kernel.
 #include "common.h"
-#include <stdlib.h>
 
 namespace aicomp {
 
@@ -160,19 +159,6 @@ __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, T
                                              int rd_off, const void* k_pool, const void* v_pool,
                                              int64_t nb0, int64_t nb1, int hkv, int kvh_next, int lane,
                                              int g4, int tile_start, int end, float cmul) {
-#ifdef EXP_LOADS_ONLY
-    {
-        uint4 x = make_uint4(0, 0, 0, 0);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { uint4 a = tile_bf16<FP8>(kr, i); x.x ^= a.x; x.y ^= a.y; x.z ^= a.z; x.w ^= a.w; }
-        if (NEXT) load_tile<FP8>(kr, k_pool, nb0, nb1, hkv, kvh_next, lane);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { uint4 a = tile_bf16<FP8>(vr, i); x.x ^= a.x; x.y ^= a.y; x.z ^= a.z; x.w ^= a.w; }
-        if (NEXT) load_tile<FP8>(vr, v_pool, nb0, nb1, hkv, kvh_next, lane);
-        st.O[0][0] += __uint_as_float(x.x ^ x.y ^ x.z ^ x.w);
-        return;
-    }
-#endif
     // ---- K tile -> LDS, then prefetch the next K tile into the same registers
 #pragma unroll
     for (int i = 0; i < 8; ++i)
@@ -795,8 +781,7 @@ int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
     }
     // one workgroup per CU measured fastest (4 waves of 16 KB in flight each already cover the
     // HBM latency; a second workgroup per CU only adds partials and start-up work)
-    int wgs = min(num_cus, SK_MAX_WAVES / NWAVES);
-    if (const char* e = getenv("AICOMP_SK_WGS")) wgs = min(atoi(e), SK_MAX_WAVES / NWAVES);  // EXPERIMENT
+    const int wgs = min(num_cus, SK_MAX_WAVES / NWAVES);
     const int group = a.hq / a.hkv;
     const int64_t slots = SK_MAX_WAVES + a.rows * a.hkv;
     StreamKParams p;

@@ -10,21 +10,28 @@
 //
 // Flops per chunk: 4 * Hq * D * (C*P + C(C+1)/2)   (QK^T and PV, causal).
 //
-// Work split   one workgroup (4 waves) per (64 query rows, sequence).  A "row" is
+// Work split   one workgroup (4 waves) per (64 or 128 query rows, sequence).  A "row" is
 //              a (position, query head) pair: with `gpack` = G heads of one KV
-//              head packed per position, the 64 rows are 64/G consecutive
-//              positions x G heads, so every K/V tile staged in LDS serves the
-//              whole GQA group.  Groups that do not divide 16 use gpack = 1.
-// K/V tiles    64 tokens (4 blocks) per step, fetched by the whole workgroup with
+//              head packed per position, the rows are consecutive positions x G
+//              heads, so every K/V tile staged in LDS serves the whole GQA group.
+//              Groups that do not divide 16 use gpack = 1.  Workgroups of one KV head
+//              are adjacent in the grid (one XCD's L2 serves them); the longest
+//              query tiles of a chunk are launched first.
+// K/V tiles    32 tokens (2 blocks) per step, fetched by the whole workgroup with
 //              coalesced 16-byte loads into registers one tile ahead, written to
-//              a double-buffered LDS tile (row stride 272 B): one barrier per tile.
-// Per wave     16 rows.  S^T = K Q^T with K rows as the A operand and the wave's
-//              16 query rows as B columns (v_mfma_f32_16x16x32_bf16); online
-//              softmax per column, lane-local except the row max (two wave
-//              shuffles); O^T += V^T P^T with V read from LDS as 16-byte row chunks
+//              a double-buffered LDS tile (row stride 272 B): one barrier per tile,
+//              35 KB of LDS per workgroup.
+// Per wave     16 or 32 rows (one or two column groups).  S^T = K Q^T with K rows as
+//              the A operand and the wave's query rows as B columns
+//              (v_mfma_f32_16x16x32_bf16); online softmax per column on the raw
+//              scores with a lazily moved max, lane-local except the row max (two
+//              lane swaps); O^T += V^T P^T with V read from LDS as 16-byte row chunks
 //              and the j-th halves picked with v_perm_b32, the same register
-//              layout as the decode kernel, so P never leaves its lane.
+//              layout as the decode kernel, so P never leaves its lane.  With two
+//              column groups every LDS operand read and permute feeds two MFMAs.
 #include "common.h"
+
+#include <type_traits>
 
 namespace aicomp {
 
@@ -36,10 +43,10 @@ namespace {
 
 constexpr int D = 128;
 constexpr int BS = 16;
-constexpr int KT = 64;                 // tokens per LDS tile
-constexpr int ROWS = 64;               // query rows per workgroup (16 per wave)
+constexpr int KT = 32;                 // tokens per LDS tile (two blocks)
+constexpr int ROWS = 64;               // query rows per workgroup and column group (16 per wave)
 constexpr int KROW = 272;              // LDS row stride in bytes (256 + 16 pad)
-constexpr int TILE_BYTES = KT * KROW;  // 17408
+constexpr int TILE_BYTES = KT * KROW;  // 8704
 constexpr float NEG_BIG = -1.0e30f;
 
 struct PrefillParams {
@@ -74,14 +81,37 @@ __device__ __forceinline__ uint4 fp8x8_to_bf16x8(uint2 r) {
     return o;
 }
 
-template <bool FP8> struct Stage;
-template <> struct Stage<false> { uint4 k[4], v[4]; };
-template <> struct Stage<true> { uint2 k[4], v[4]; };
+// max over lanes l and l^16 (l^32): gfx950's lane-swap instructions, no LDS round trip.
+// v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of
+// its second; with both operands holding x, every lane ends up with its own value in one
+// result and its partner's in the other.
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float xor16_max(float x) {
+    const u32x2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xor32_max(float x) {
+    const u32x2_t r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
 
-template <bool FP8>
-__global__ void __launch_bounds__(256, 2)
+template <bool FP8> struct Stage;
+template <> struct Stage<false> { uint4 k[KT / 16], v[KT / 16]; };
+template <> struct Stage<true> { uint2 k[KT / 16], v[KT / 16]; };
+
+// R = 16-row column groups per wave (1 or 2).  With R = 2 every K and V operand read from LDS
+// (and every V permute) feeds two MFMAs, and the two groups' softmax chains are independent, so
+// LDS traffic and permute work per flop halve and the scheduler has two chains to interleave.
+template <bool FP8, int R>
+__global__ void __launch_bounds__(256, R == 1 ? 3 : 2)
 paged_prefill_mfma_kernel(PrefillParams p) {
+    // Grid: x = head group (fastest: the workgroups of one KV head land on one XCD and share its
+    // L2 copy of that head's K/V), y = query tile, longest first (the last tile of a chunk sees
+    // the most keys, so it is started first), z = sequence.
+    constexpr int WROWS = 16 * R;              // rows per wave
     const int seq = blockIdx.z;
+    const int hgroup = blockIdx.x;
+    const int qtile = gridDim.y - 1 - blockIdx.y;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -91,49 +121,73 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     const int n = p.cu_q_lens[seq + 1] - q_begin;
     const int ctx = min(p.context_lens[seq], p.max_blocks * BS);
     const int prior = ctx - n;
-    const int pos_per_wg = ROWS / p.gpack;
-    const int q0 = blockIdx.x * pos_per_wg;
+    const int pos_per_wg = ROWS * R / p.gpack;
+    const int q0 = qtile * pos_per_wg;
     if (q0 >= n || n <= 0 || prior < 0) return;
 
-    // rows of this lane's column: row = 16w + r16 -> (position, head)
-    const int row = 16 * w + r16;
-    const int qpos = q0 + row / p.gpack;
-    const int head = blockIdx.y * p.gpack + row % p.gpack;
-    const int kvh = (blockIdx.y * p.gpack) / p.group;          // workgroup-uniform
-    const bool row_valid = qpos < n;
-    const int qabs = row_valid ? prior + qpos : ctx - 1;        // padded rows: computed, never stored
+    // rows of this lane's columns: row = WROWS*w + 16c + r16 -> (position, head)
+    const int kvh = (hgroup * p.gpack) / p.group;          // workgroup-uniform
+    int qpos[R], head[R], qabs[R];
+    bool row_valid[R];
+#pragma unroll
+    for (int c = 0; c < R; ++c) {
+        const int row = WROWS * w + 16 * c + r16;
+        qpos[c] = q0 + row / p.gpack;
+        head[c] = hgroup * p.gpack + row % p.gpack;
+        row_valid[c] = qpos[c] < n;
+        qabs[c] = row_valid[c] ? prior + qpos[c] : ctx - 1;    // padded rows: computed, never stored
+    }
     // last key any row of this wave / workgroup may see (exclusive)
-    const int wave_kv_end = min(ctx, prior + q0 + (16 * w + 15) / p.gpack + 1);
-    const int wave_kv_min = prior + q0 + (16 * w) / p.gpack;    // smallest qabs in the wave (if valid)
+    const int wave_kv_end = min(ctx, prior + q0 + (WROWS * w + WROWS - 1) / p.gpack + 1);
+    const int wave_kv_min = prior + q0 + (WROWS * w) / p.gpack;    // smallest qabs in the wave (if valid)
     const int kv_end = min(ctx, prior + q0 + pos_per_wg);
     const int ntiles = (kv_end + KT - 1) / KT;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [2][K tile | V tile]
 
     // Q as the B operand: column = this lane's row, k-slots = dims 32s + 8*g4 ..
-    bf16x8_t qf[4];
-    {
+    bf16x8_t qf[R][4];
+#pragma unroll
+    for (int c = 0; c < R; ++c) {
         const uint4* qp = (const uint4*)((const bf16_t*)p.query +
-                                         ((int64_t)(q_begin + min(qpos, n - 1)) * p.hq + head) * D + 8 * g4);
+                                         ((int64_t)(q_begin + min(qpos[c], n - 1)) * p.hq + head[c]) * D + 8 * g4);
 #pragma unroll
-        for (int s = 0; s < 4; ++s) qf[s] = __builtin_bit_cast(bf16x8_t, qp[s * 4]);
+        for (int s = 0; s < 4; ++s) qf[c][s] = __builtin_bit_cast(bf16x8_t, qp[s * 4]);
     }
-    const float cmul = p.qk_mul * (FP8 ? p.k_scale[kvh] : 1.f);
-
-    float m = NEG_BIG, lsum = 0.f;
-    f32x4_t O[8];
+    // log2(e) * scale * k_scale.  The softmax below tracks the max of the raw scores, which needs
+    // a positive multiplier: a negative one (a negative k_scale) moves its sign into Q.
+    float cmul = p.qk_mul * (FP8 ? p.k_scale[kvh] : 1.f);
+    if (cmul < 0.f) {
+        cmul = -cmul;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) O[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int c = 0; c < R; ++c)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                uint4 u = __builtin_bit_cast(uint4, qf[c][s]);
+                u.x ^= 0x80008000u; u.y ^= 0x80008000u; u.z ^= 0x80008000u; u.w ^= 0x80008000u;
+                qf[c][s] = __builtin_bit_cast(bf16x8_t, u);
+            }
+    }
+
+    const float lazy_thr = 8.f / cmul;          // +inf for a zero multiplier: every P is 1
+    float m[R], lsum[R];
+    f32x4_t O[R][8];
+#pragma unroll
+    for (int c = 0; c < R; ++c) {
+        m[c] = NEG_BIG; lsum[c] = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) O[c][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
 
     typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
     const_i32_ptr table = (const_i32_ptr)(p.block_table + (int64_t)seq * p.block_table_stride);
 
-    // global -> registers: load i of the tile is block 4t + i (16 tokens x 16 chunks = 256 lanes)
+    // global -> registers: load i of the tile is block (KT/16)*t + i (16 tokens x 16 chunks = 256 lanes)
     Stage<FP8> st;
     auto fetch = [&](int t) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int bi = 4 * t + i;
+        for (int i = 0; i < KT / 16; ++i) {
+            const int bi = (KT / 16) * t + i;
             int b = bi < p.max_blocks ? table[bi] : 0;
             const int64_t blk = b < 0 ? 0 : (b >= p.num_blocks ? p.num_blocks - 1 : (int64_t)b);
             const int64_t off = (blk * p.hkv + kvh) * (BS * D / 8) + tid;
@@ -152,7 +206,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         unsigned char* kb = lds + buf * 2 * TILE_BYTES;
         unsigned char* vb = kb + TILE_BYTES;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < KT / 16; ++i) {
             const int tok_local = 16 * i + (tid >> 4);
             const int off = tok_local * KROW + (tid & 15) * 16;
             uint4 kk, vv;
@@ -176,87 +230,127 @@ paged_prefill_mfma_kernel(PrefillParams p) {
 
         const unsigned char* kb = lds + buf * 2 * TILE_BYTES;
         const unsigned char* vb = kb + TILE_BYTES;
+        const int sub_start = t * KT;
+        if (sub_start >= wave_kv_end) continue;                        // wave-uniform: above the diagonal
+
+        // ---- S^T = K Q^T: each K operand read feeds the R column groups
+        f32x4_t s0[R], s1[R];
 #pragma unroll
-        for (int sub = 0; sub < 2; ++sub) {
-            const int sub_start = t * KT + sub * 32;
-            if (sub_start >= wave_kv_end) continue;                    // wave-uniform: above the diagonal
-            f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+        for (int c = 0; c < R; ++c) { s0[c] = f32x4_t{0.f, 0.f, 0.f, 0.f}; s1[c] = f32x4_t{0.f, 0.f, 0.f, 0.f}; }
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const uint4 a0 = *(const uint4*)(kb + sub * 32 * KROW + rd_k + s * 64);
-                const uint4 a1 = *(const uint4*)(kb + (sub * 32 + 16) * KROW + rd_k + s * 64);
-                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a0), qf[s], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a1), qf[s], s1, 0, 0, 0);
+        for (int s = 0; s < 4; ++s) {
+            const bf16x8_t a0 = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kb + rd_k + s * 64));
+            const bf16x8_t a1 = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kb + 16 * KROW + rd_k + s * 64));
+#pragma unroll
+            for (int c = 0; c < R; ++c) {
+                s0[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[c][s], s0[c], 0, 0, 0);
+                s1[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qf[c][s], s1[c], 0, 0, 0);
             }
-            float sc[8];
+        }
+        // Online softmax on the raw scores: the score multiplier is folded into the exponent's
+        // fused multiply-add and the running max stays in raw units.  The max is only moved when a
+        // row's new maximum exceeds it by more than 2^8 after scaling: until then P is at most
+        // 256, exact enough in bf16 and f32, and the accumulators need no rescale.  Only tiles that
+        // cross the diagonal pay for the mask.
+        const bool need_mask = sub_start + KT - 1 > wave_kv_min;       // wave-uniform
+        bf16x8_t pf[R];
+        float alpha[R];
+        auto softmax = [&](auto mask_tag) {
+            constexpr bool MASK = decltype(mask_tag)::value;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) { sc[i] = s0[i] * cmul; sc[4 + i] = s1[i] * cmul; }
-            const bool need_mask = sub_start + 31 > wave_kv_min;       // wave-uniform
-            if (need_mask) {
+            for (int c = 0; c < R; ++c) {
+                float sc[8];
+                bool dead[8];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { sc[i] = s0[c][i]; sc[4 + i] = s1[c][i]; }
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
-                    const int tok = sub_start + 16 * (k >> 2) + 4 * (k & 3) + g4;
-                    if (tok > qabs) sc[k] = NEG_BIG;
+                    dead[k] = MASK && sub_start + 16 * (k >> 2) + 4 * (k & 3) + g4 > qabs[c];
+                    if (MASK && dead[k]) sc[k] = NEG_BIG;
                 }
-            }
-            float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
-                             fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-            mx = fmaxf(mx, __shfl_xor(mx, 16));
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float m_new = fmaxf(m, mx);
-            const float alpha = exp2f(m - m_new);
-            float pr[8], psum = 0.f;
+                float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
+                                 fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+                mx = xor16_max(mx);
+                mx = xor32_max(mx);
+                alpha[c] = 1.f;
+                if (mx - m[c] > lazy_thr) {
+                    alpha[c] = __builtin_amdgcn_exp2f((m[c] - mx) * cmul);
+                    m[c] = mx;
+                }
+                const float bias = -m[c] * cmul;
+                float pr[8], psum = 0.f;
 #pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                pr[k] = exp2f(sc[k] - m_new);
-                if (need_mask && sc[k] == NEG_BIG) pr[k] = 0.f;
-                psum += pr[k];
+                for (int k = 0; k < 8; ++k) {
+                    pr[k] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[k], cmul, bias));
+                    if (MASK && dead[k]) pr[k] = 0.f;
+                    psum += pr[k];
+                }
+                lsum[c] = lsum[c] * alpha[c] + psum;
+                uint4 pw;
+                pw.x = pack_bf16(pr[0], pr[1]); pw.y = pack_bf16(pr[2], pr[3]);
+                pw.z = pack_bf16(pr[4], pr[5]); pw.w = pack_bf16(pr[6], pr[7]);
+                pf[c] = __builtin_bit_cast(bf16x8_t, pw);
             }
-            lsum = lsum * alpha + psum;
-            m = m_new;
-            if (__any(alpha != 1.f)) {
+        };
+        if (need_mask) softmax(std::true_type{}); else softmax(std::false_type{});
 #pragma unroll
-                for (int j = 0; j < 8; ++j) O[j] *= alpha;
+        for (int c = 0; c < R; ++c) {
+            if (__any(alpha[c] != 1.f)) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) O[c][j] *= alpha[c];
             }
-            uint4 pw;
-            pw.x = pack_bf16(pr[0], pr[1]); pw.y = pack_bf16(pr[2], pr[3]);
-            pw.z = pack_bf16(pr[4], pr[5]); pw.w = pack_bf16(pr[6], pr[7]);
-            const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pw);
+        }
 
-            uint4 vv[8];
+        // ---- O^T += V^T P^T: each permuted V operand feeds the R column groups
+        uint4 vv[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
-                vv[i] = *(const uint4*)(vb + (sub * 32 + 4 * i) * KROW + rd_v);
+        for (int i = 0; i < 8; ++i) vv[i] = *(const uint4*)(vb + 4 * i * KROW + rd_v);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
-                const uint32_t* v0 = (const uint32_t*)&vv[0];
-                uint4 a;
-                a.x = __builtin_amdgcn_perm(v0[4 * 1 + (j >> 1)], v0[4 * 0 + (j >> 1)], sel);
-                a.y = __builtin_amdgcn_perm(v0[4 * 3 + (j >> 1)], v0[4 * 2 + (j >> 1)], sel);
-                a.z = __builtin_amdgcn_perm(v0[4 * 5 + (j >> 1)], v0[4 * 4 + (j >> 1)], sel);
-                a.w = __builtin_amdgcn_perm(v0[4 * 7 + (j >> 1)], v0[4 * 6 + (j >> 1)], sel);
-                O[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), pf, O[j], 0, 0, 0);
-            }
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+            const uint32_t* v0 = (const uint32_t*)&vv[0];
+            uint4 a;
+            a.x = __builtin_amdgcn_perm(v0[4 * 1 + (j >> 1)], v0[4 * 0 + (j >> 1)], sel);
+            a.y = __builtin_amdgcn_perm(v0[4 * 3 + (j >> 1)], v0[4 * 2 + (j >> 1)], sel);
+            a.z = __builtin_amdgcn_perm(v0[4 * 5 + (j >> 1)], v0[4 * 4 + (j >> 1)], sel);
+            a.w = __builtin_amdgcn_perm(v0[4 * 7 + (j >> 1)], v0[4 * 6 + (j >> 1)], sel);
+#pragma unroll
+            for (int c = 0; c < R; ++c)
+                O[c][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), pf[c], O[c][j], 0, 0, 0);
         }
     }
 
-    // lane (row r16 of the wave, g4) holds O^T[dim 32*g4 + 8*i + j][row] in O[j][i]
-    lsum += __shfl_xor(lsum, 16);
-    lsum += __shfl_xor(lsum, 32);
-    if (row_valid) {
-        const float inv = (lsum > 0.f ? 1.f / lsum : 0.f) * (FP8 ? p.v_scale[kvh] : 1.f);
-        bf16_t* o = (bf16_t*)p.out + ((int64_t)(q_begin + qpos) * p.hq + head) * D + 32 * g4;
+    // lane (row r16 of column group c, g4) holds O^T[dim 32*g4 + 8*i + j][row] in O[c][j][i]
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            uint4 pk;
-            pk.x = pack_bf16(O[0][i] * inv, O[1][i] * inv);
-            pk.y = pack_bf16(O[2][i] * inv, O[3][i] * inv);
-            pk.z = pack_bf16(O[4][i] * inv, O[5][i] * inv);
-            pk.w = pack_bf16(O[6][i] * inv, O[7][i] * inv);
-            *(uint4*)(o + 8 * i) = pk;
+    for (int c = 0; c < R; ++c) {
+        float l = lsum[c];
+        l += __shfl_xor(l, 16);
+        l += __shfl_xor(l, 32);
+        if (row_valid[c]) {
+            const float inv = (l > 0.f ? 1.f / l : 0.f) * (FP8 ? p.v_scale[kvh] : 1.f);
+            bf16_t* o = (bf16_t*)p.out + ((int64_t)(q_begin + qpos[c]) * p.hq + head[c]) * D + 32 * g4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                uint4 pk;
+                pk.x = pack_bf16(O[c][0][i] * inv, O[c][1][i] * inv);
+                pk.y = pack_bf16(O[c][2][i] * inv, O[c][3][i] * inv);
+                pk.z = pack_bf16(O[c][4][i] * inv, O[c][5][i] * inv);
+                pk.w = pack_bf16(O[c][6][i] * inv, O[c][7][i] * inv);
+                *(uint4*)(o + 8 * i) = pk;
+            }
         }
     }
+}
+
+template <bool FP8, int R>
+static void launch_prefill_variant(const PrefillParams& p, dim3 grid, size_t lds_bytes, hipStream_t stream) {
+    static bool once = false;
+    if (!once) {
+        hipFuncSetAttribute((const void*)paged_prefill_mfma_kernel<FP8, R>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        once = true;
+    }
+    hipLaunchKernelGGL((paged_prefill_mfma_kernel<FP8, R>), grid, dim3(256), lds_bytes, stream, p);
 }
 
 }  // namespace
@@ -281,29 +375,18 @@ int launch_prefill_mfma(const DecodeArgs& a, int max_q_len) {
     p.gpack = (16 % p.group == 0) ? p.group : 1;      // heads of one KV head packed per position
     p.qk_mul = a.scale * LOG2E;
     p.k_scale = a.k_scale; p.v_scale = a.v_scale;
-    const int pos_per_wg = ROWS / p.gpack;
+    // two column groups per wave (128 rows per workgroup) once a chunk has that many rows
+    const int R = (int64_t)max_q_len * p.gpack >= 2 * ROWS ? 2 : 1;
+    const int pos_per_wg = ROWS * R / p.gpack;
     const int qtiles = (max_q_len + pos_per_wg - 1) / pos_per_wg;
-    AICOMP_REQUIRE(qtiles <= 65535 * 32768 && a.hq / p.gpack <= 65535, AICOMP_KV_EINVAL,
-                   "paged_prefill_attn: grid too large");
-    dim3 grid((unsigned)qtiles, (unsigned)(a.hq / p.gpack), (unsigned)a.num_seqs);
+    AICOMP_REQUIRE(qtiles <= 65535, AICOMP_KV_EINVAL, "paged_prefill_attn: grid too large");
+    dim3 grid((unsigned)(a.hq / p.gpack), (unsigned)qtiles, (unsigned)a.num_seqs);
     const size_t lds_bytes = 4 * TILE_BYTES;   // double-buffered K and V tiles
-    if (a.kv_dtype == AICOMP_KV_FP8_E4M3) {
-        static bool once_fp8 = false;
-        if (!once_fp8) {
-            hipFuncSetAttribute((const void*)paged_prefill_mfma_kernel<true>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-            once_fp8 = true;
-        }
-        hipLaunchKernelGGL(paged_prefill_mfma_kernel<true>, grid, dim3(256), lds_bytes, a.stream, p);
-    } else {
-        static bool once = false;
-        if (!once) {
-            hipFuncSetAttribute((const void*)paged_prefill_mfma_kernel<false>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-            once = true;
-        }
-        hipLaunchKernelGGL(paged_prefill_mfma_kernel<false>, grid, dim3(256), lds_bytes, a.stream, p);
-    }
+    const bool fp8 = a.kv_dtype == AICOMP_KV_FP8_E4M3;
+    if (fp8 && R == 2) launch_prefill_variant<true, 2>(p, grid, lds_bytes, a.stream);
+    else if (fp8) launch_prefill_variant<true, 1>(p, grid, lds_bytes, a.stream);
+    else if (R == 2) launch_prefill_variant<false, 2>(p, grid, lds_bytes, a.stream);
+    else launch_prefill_variant<false, 1>(p, grid, lds_bytes, a.stream);
     AICOMP_HIP_LAUNCH_CHECK();
     return AICOMP_KV_OK;
 }
