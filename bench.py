@@ -107,6 +107,18 @@ def run_decode_config(name, steps, warmup, dev):
         append_only()
     a1.record()
     torch.cuda.synchronize()
+    # cold figure: the decode call right after 1 GiB of unrelated writes has gone through L2 and
+    # the memory-side cache (the steady-state loop above re-reads the same pool every step)
+    cold = []
+    for _ in range(8):
+        filler.fill_(2)
+        c0, c1 = _events(2)
+        c0.record()
+        ops.paged_decode_attn(outd, qd, w.k_pool, w.v_pool, btd, cld, w.scale, w.k_scale, w.v_scale)
+        c1.record()
+        cold.append((c0, c1))
+    torch.cuda.synchronize()
+    t_cold = statistics.median(a.elapsed_time(b) for a, b in cold) * 1e-3
     del filler
     t_app = a0.elapsed_time(a1) / 20 * 1e-3
     t_pre = statistics.mean(e[1].elapsed_time(e[2]) for e in evs) * 1e-3 if npre else 0.0
@@ -120,6 +132,7 @@ def run_decode_config(name, steps, warmup, dev):
         "decode_GBs": w.decode_kv_bytes() / t_dec / 1e9,
         "decode_frac_hbm_peak": w.decode_kv_bytes() / t_dec / 1e9 / HBM_PEAK_GBS,
         "decode_tokens_per_s": (S - npre) / t_dec,
+        "decode_cold_us": t_cold * 1e6, "decode_cold_GBs": w.decode_kv_bytes() / t_cold / 1e9,
         "partition_size": ops.decode_partition_size(S - npre, w.shape.num_q_heads, w.shape.num_kv_heads,
                                                     w.shape.head_dim, w.shape.block_size, btd.shape[1],
                                                     qd.dtype, w.k_pool.dtype),
@@ -130,6 +143,42 @@ def run_decode_config(name, steps, warmup, dev):
                     "prefill_TFLOPs": w.prefill_flops() / t_pre / 1e12,
                     "prefill_frac_mfma_peak": w.prefill_flops() / t_pre / 1e12 / MFMA_BF16_PEAK_TFLOPS})
     return res, w
+
+
+def planner_bench(dev):
+    """Host cost of planning one decode step for the headline batch (64 sequences, contexts
+    uniform in [512, 4096]): free-list growth, block table, context lengths and slots packed
+    into one pinned buffer and copied with one asynchronous transfer.  One plan serves every
+    layer of a model step."""
+    import numpy as np
+    import torch
+    from aicomp_amd.block_manager import StepPlanner
+    rng = np.random.default_rng(0)
+    pl = StepPlanner(num_blocks=12000, max_seqs=64, max_seq_len=4608, max_num_batched_tokens=8192,
+                     prefill_chunk=512, device=dev)
+    for i in range(64):
+        pl.add_request(i, int(rng.integers(512, 4097)))
+    plan = pl.schedule()
+    while plan.num_prefill_seqs:
+        plan = pl.schedule()
+    torch.cuda.synchronize()
+    n = 200
+    t0 = time.perf_counter()
+    for _ in range(n):
+        plan = pl.schedule()
+    host = (time.perf_counter() - t0) / n
+    torch.cuda.synchronize()
+    return {"decode_plan_host_us": host * 1e6, "seqs": plan.num_seqs,
+            "h2d_bytes_per_plan": int(8 * plan.total_new_tokens + 4 * (plan.block_table.numel() + 2 * plan.num_seqs + 1)),
+            "note": "StepPlanner.schedule() per decode step, including the enqueue of its one H2D copy"}
+
+
+def device_info():
+    import torch
+    p = torch.cuda.get_device_properties(0)
+    return {"name": p.name, "arch": getattr(p, "gcnArchName", ""), "compute_units": p.multi_processor_count,
+            "clock_mhz": getattr(p, "clock_rate", 0) / 1e3, "hbm_gib": round(p.total_memory / 2**30, 1),
+            "hbm_peak_GBs_used": HBM_PEAK_GBS, "mfma_bf16_peak_TFLOPs_used": MFMA_BF16_PEAK_TFLOPS}
 
 
 def profile_target(which, steps, warmup, dev):
@@ -275,6 +324,10 @@ def main():
                      "avg_launch_us": main_res["decode_us"]},
         "append": {"us": main_res["append_us"], "GB/s": main_res["append_GBs"],
                    "bytes": main_res["append_bytes"]},
+        "decode_cold": {"us": main_res["decode_cold_us"], "GB/s": main_res["decode_cold_GBs"],
+                        "note": "decode call timed right after 1 GiB of unrelated writes"},
+        "device": device_info(),
+        "step_planner": planner_bench(dev),
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(w)

@@ -1,0 +1,106 @@
+"""Continuous batching end to end: planner -> append / prefill / decode kernels vs the oracle.
+
+Every sequence keeps its own K/V history on the host; after each planned step the rows the
+kernels produced are compared with textbook attention over that history (float64), and the
+pool is read back through the plan's block table to check the append bit for bit.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from aicomp_amd.block_manager import StepPlanner, paged_attention_step
+from oracle import paged_kv_oracle as orc
+from helpers import assert_close_attn, raw, to_f64
+
+pytestmark = pytest.mark.gpu
+BF16_ATOL, BF16_RTOL = 1e-2, 2e-2
+
+
+def run_serving(device, kv_dtype, steps, seed, num_blocks=96, hq=8, hkv=2, d=128):
+    g = torch.Generator().manual_seed(seed)
+    rng = np.random.default_rng(seed)
+    p = StepPlanner(num_blocks=num_blocks, max_seqs=12, max_seq_len=400, max_num_batched_tokens=256,
+                    prefill_chunk=96, device=device)
+    fp8 = kv_dtype == torch.float8_e4m3fn
+    # pools start non-finite: nothing beyond a context may leak into a result
+    k_pool = torch.full((num_blocks, hkv, 16, d), float("nan"), dtype=torch.bfloat16, device=device).to(kv_dtype)
+    v_pool = torch.full((num_blocks, hkv, 16, d), float("nan"), dtype=torch.bfloat16, device=device).to(kv_dtype)
+    ks = vs = None
+    if fp8:
+        ks = torch.full((hkv,), 3.0 / 448, dtype=torch.float32, device=device)
+        vs = torch.full((hkv,), 2.5 / 448, dtype=torch.float32, device=device)
+    scale = 1 / math.sqrt(d)
+    hist = {}                      # seq -> (K [L,Hkv,D] float64 as stored, V likewise)
+    nxt = checked = pre_rows = dec_rows = 0
+    for step in range(steps):
+        if rng.random() < 0.45:
+            p.add_request(nxt, int(rng.integers(1, 220)), int(rng.integers(1, 40)))
+            nxt += 1
+        for sid in p.completed():
+            p.finish(sid)
+            hist.pop(sid, None)
+        plan = p.schedule()
+        if plan is None:
+            continue
+        for sid in plan.preempted:
+            hist.pop(sid, None)
+        T = plan.total_new_tokens
+        q = torch.randn(T, hq, d, generator=g).to(torch.bfloat16).to(device)
+        k = (torch.randn(T, hkv, d, generator=g) * 0.5).to(torch.bfloat16).to(device)
+        v = (torch.randn(T, hkv, d, generator=g) * 0.5).to(torch.bfloat16).to(device)
+        out = torch.full((T, hq, d), float("nan"), dtype=torch.bfloat16, device=device)
+        print(f"step {step}: {plan.num_prefill_seqs} chunks + {plan.num_decode_seqs} decode rows, T={T}", flush=True)
+        paged_attention_step(plan, out, q, k, v, k_pool, v_pool, scale, ks, vs)
+        torch.cuda.synchronize()
+        # what the pool now holds for these rows (quantised for fp8), as float64
+        if fp8:
+            kq = orc.e4m3_bits_to_f32(orc.f32_to_e4m3_bits(k.float().cpu().numpy() / ks.cpu().numpy()[None, :, None]))
+            vq = orc.e4m3_bits_to_f32(orc.f32_to_e4m3_bits(v.float().cpu().numpy() / vs.cpu().numpy()[None, :, None]))
+            k_st = kq.astype(np.float64) * ks.cpu().numpy()[None, :, None]
+            v_st = vq.astype(np.float64) * vs.cpu().numpy()[None, :, None]
+        else:
+            k_st, v_st = to_f64(k), to_f64(v)
+        kp_raw, vp_raw = raw(k_pool), raw(v_pool)
+        cu = plan.host_cu_q_lens
+        got = to_f64(out)
+        qf = to_f64(q)
+        for r, sid in enumerate(plan.seq_ids):
+            n = int(plan.new_lens[r])
+            hk, hv = hist.get(sid, (np.zeros((0, hkv, d)), np.zeros((0, hkv, d))))
+            prior = hk.shape[0]
+            hk = np.concatenate([hk, k_st[cu[r]:cu[r + 1]]])
+            hv = np.concatenate([hv, v_st[cu[r]:cu[r + 1]]])
+            hist[sid] = (hk, hv)
+            L = prior + n
+            assert plan.host_context_lens[r] == L
+            want = orc.attend_contiguous(qf[cu[r]:cu[r + 1]], hk, hv, scale, prior=prior)
+            assert_close_attn(got[cu[r]:cu[r + 1]], want, BF16_ATOL, BF16_RTOL,
+                              f"step {step} seq {sid} (prior {prior}, new {n})")
+            # the append, bit for bit, through the block table
+            if not fp8:
+                gk = orc.gather_context(kp_raw, plan.host_block_table[r], L)
+                assert (gk[prior:] == raw(k[cu[r]:cu[r + 1]])).all()
+                gv = orc.gather_context(vp_raw, plan.host_block_table[r], L)
+                assert (gv[prior:] == raw(v[cu[r]:cu[r + 1]])).all()
+            checked += 1
+            pre_rows += n > 1
+            dec_rows += n == 1
+    return checked, pre_rows, dec_rows, p
+
+
+def test_serving_loop_bf16(device):
+    checked, pre, dec, p = run_serving(device, torch.bfloat16, steps=60, seed=0)
+    assert pre >= 10 and dec >= 100
+
+
+def test_serving_loop_with_preemption(device):
+    # 40 blocks = 640 tokens for up to 12 sequences of up to ~260 tokens: the pool runs dry
+    checked, pre, dec, p = run_serving(device, torch.bfloat16, steps=70, seed=1, num_blocks=40)
+    assert p.num_preemptions > 0 and dec >= 100
+
+
+def test_serving_loop_fp8(device):
+    checked, pre, dec, p = run_serving(device, torch.float8_e4m3fn, steps=40, seed=2)
+    assert pre >= 5 and dec >= 50
