@@ -86,6 +86,52 @@ int aicomp_kv_append(const void* key, const void* value, int64_t kv_token_stride
                             (hipStream_t)stream);
 }
 
+int aicomp_rope_kv_append(const void* q_in, void* q_out, int64_t q_token_stride,
+                          int64_t q_head_stride, int64_t qo_token_stride, int64_t qo_head_stride,
+                          const void* key, const void* value, int64_t kv_token_stride,
+                          int64_t kv_head_stride, const void* cos, const void* sin,
+                          int64_t table_stride, int64_t table_rows, const int64_t* positions,
+                          void* k_pool, void* v_pool, const int64_t* slot_mapping,
+                          int64_t num_tokens, int num_q_heads, int num_kv_heads, int head_dim,
+                          int block_size, int64_t num_blocks, int in_dtype, int pool_dtype,
+                          const float* k_scale, const float* v_scale, void* stream) {
+    AICOMP_REQUIRE(num_tokens >= 0, AICOMP_KV_EINVAL, "rope_kv_append: negative token count");
+    if (num_tokens == 0) return AICOMP_KV_OK;
+    AICOMP_REQUIRE(q_in && q_out && key && value && cos && sin && k_pool && v_pool && slot_mapping,
+                   AICOMP_KV_EINVAL, "rope_kv_append: null pointer");
+    AICOMP_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0 && block_size > 0 &&
+                   num_blocks > 0 && table_rows > 0, AICOMP_KV_EINVAL,
+                   "rope_kv_append: bad sizes (Hq %d, Hkv %d, D %d, BS %d, blocks %lld, table rows %lld)",
+                   num_q_heads, num_kv_heads, head_dim, block_size, (long long)num_blocks,
+                   (long long)table_rows);
+    AICOMP_REQUIRE(in_dtype == AICOMP_KV_F32 || in_dtype == AICOMP_KV_BF16, AICOMP_KV_EUNSUPPORTED,
+                   "rope_kv_append: inputs must be float32 or bfloat16 (got %d)", in_dtype);
+    AICOMP_REQUIRE(pool_dtype == in_dtype || pool_dtype == AICOMP_KV_FP8_E4M3, AICOMP_KV_EUNSUPPORTED,
+                   "rope_kv_append: pool type %d must be the input type %d or fp8-e4m3", pool_dtype,
+                   in_dtype);
+    AICOMP_REQUIRE(pool_dtype != AICOMP_KV_FP8_E4M3 || (k_scale && v_scale), AICOMP_KV_EINVAL,
+                   "rope_kv_append: an fp8 pool needs k_scale and v_scale");
+    AICOMP_REQUIRE(head_dim % 16 == 0, AICOMP_KV_EUNSUPPORTED,
+                   "rope_kv_append: head_dim %d is not a multiple of 16", head_dim);
+    const int64_t v = 16 / dtype_size(in_dtype);       // elements per 16 bytes
+    AICOMP_REQUIRE(q_head_stride >= head_dim && qo_head_stride >= head_dim &&
+                   kv_head_stride >= head_dim && table_stride >= head_dim && q_token_stride >= 0 &&
+                   qo_token_stride >= 0 && kv_token_stride >= 0, AICOMP_KV_EINVAL,
+                   "rope_kv_append: strides overlap rows of %d elements", head_dim);
+    AICOMP_REQUIRE(q_token_stride % v == 0 && q_head_stride % v == 0 && qo_token_stride % v == 0 &&
+                   qo_head_stride % v == 0 && kv_token_stride % v == 0 && kv_head_stride % v == 0 &&
+                   table_stride % v == 0, AICOMP_KV_EUNSUPPORTED,
+                   "rope_kv_append: strides must be multiples of %lld elements (16 bytes)", (long long)v);
+    AICOMP_REQUIRE(((uintptr_t)q_in | (uintptr_t)q_out | (uintptr_t)key | (uintptr_t)value |
+                    (uintptr_t)cos | (uintptr_t)sin | (uintptr_t)k_pool | (uintptr_t)v_pool) % 16 == 0,
+                   AICOMP_KV_EUNSUPPORTED, "rope_kv_append: pointers must be 16-byte aligned");
+    return launch_rope_kv_append(q_in, q_out, q_token_stride, q_head_stride, qo_token_stride,
+                                 qo_head_stride, key, value, kv_token_stride, kv_head_stride, cos, sin,
+                                 table_stride, table_rows, positions, k_pool, v_pool, slot_mapping,
+                                 num_tokens, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks,
+                                 in_dtype, pool_dtype, k_scale, v_scale, (hipStream_t)stream);
+}
+
 int aicomp_paged_decode_partition_size(int batch, int num_q_heads, int num_kv_heads, int head_dim,
                                        int block_size, int max_blocks_per_seq, int q_dtype,
                                        int kv_dtype) {

@@ -171,5 +171,12 @@ int launch_kv_append_last(const void* key, const void* value, int64_t token_stri
                           int pool_dtype, const float* k_scale, const float* v_scale,
                           hipStream_t stream);
 int launch_split_reduce(const DecodeArgs& a);
+int launch_rope_kv_append(const void* q_in, void* q_out, int64_t q_ts, int64_t q_hs, int64_t qo_ts,
+                          int64_t qo_hs, const void* key, const void* value, int64_t kv_ts,
+                          int64_t kv_hs, const void* cos_tab, const void* sin_tab, int64_t tab_stride,
+                          int64_t tab_rows, const int64_t* positions, void* k_pool, void* v_pool,
+                          const int64_t* slot_mapping, int64_t num_tokens, int hq, int hkv, int d, int bs,
+                          int64_t num_blocks, int in_dtype, int pool_dtype, const float* k_scale,
+                          const float* v_scale, hipStream_t stream);
 
 }  // namespace aicomp

@@ -221,3 +221,77 @@ def paged_prefill_attn(out: torch.Tensor, query: torch.Tensor, k_pool: torch.Ten
                                        _stream(query))
     _lib.check(rc, lib)
     return out
+
+
+def rotary_tables(inv_freq: torch.Tensor, num_positions: int, dtype: torch.dtype,
+                  attention_scaling: float = 1.0, device=None):
+    """cos / sin tables ``[num_positions, D]`` the way the reference's rotary module builds them
+    per call (compiler_fx/modeling_llama.py:150-168): ``freqs = position * inv_freq`` in
+    float32, ``emb = cat(freqs, freqs)``, ``cos(emb) * attention_scaling`` cast to the
+    tensor type.  Built once; ``rope_kv_append`` indexes them by position.
+    """
+    device = inv_freq.device if device is None else device
+    inv = inv_freq.to(device=device, dtype=torch.float32)
+    pos = torch.arange(num_positions, device=device, dtype=torch.float32)
+    freqs = (inv[:, None] @ pos[None, :]).transpose(0, 1)          # the reference's matmul form
+    emb = torch.cat((freqs, freqs), dim=-1)
+    cos = (emb.cos() * attention_scaling).to(dtype).contiguous()
+    sin = (emb.sin() * attention_scaling).to(dtype).contiguous()
+    return cos, sin
+
+
+def rope_kv_append(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, cos: torch.Tensor,
+                   sin: torch.Tensor, positions: Optional[torch.Tensor], k_pool: torch.Tensor,
+                   v_pool: torch.Tensor, slot_mapping: torch.Tensor,
+                   k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
+                   query_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Rotate ``query [T, Hq, D]`` and ``key [T, Hkv, D]`` by their positions and append the rotated
+    key and ``value`` to the pools, in one launch.
+
+    ``cos`` / ``sin`` are ``[P, D]`` tables of the query dtype; ``positions [T]`` int64 selects the
+    row of each token (``None``: row t, i.e. per-token cos/sin as the reference passes them).
+    Returns the rotated query (``query_out``, by default ``query`` itself, in place).  The three
+    inputs may be views into one fused QKV projection output (last dimension contiguous).
+    """
+    lib = _lib.load()
+    _req(query.is_cuda, "tensors must live on a ROCm device (there is no CPU path)")
+    nb, hkv, bs, d = _check_pools(k_pool, v_pool)
+    out = query if query_out is None else query_out
+    _req(query.dim() == 3 and key.dim() == 3 and value.shape == key.shape and out.shape == query.shape,
+         "query/query_out must be [T, Hq, D], key/value [T, Hkv, D]")
+    T, hq, dq = query.shape
+    _req(key.shape == (T, hkv, d) and dq == d,
+         f"key/value {tuple(key.shape)} and query {tuple(query.shape)} do not match pools {tuple(k_pool.shape)}")
+    _req(key.dtype == query.dtype and value.dtype == query.dtype and out.dtype == query.dtype,
+         "query, key, value and query_out must share one dtype")
+    _req(query.dtype in (torch.float32, torch.bfloat16), f"unsupported input dtype {query.dtype}")
+    for t, n in ((query, "query"), (out, "query_out"), (key, "key"), (value, "value")):
+        _req(t.stride(2) == 1, f"{n}: last dimension must be contiguous")
+    _req(key.stride() == value.stride(), "key and value must have equal strides")
+    _req(cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] == d and cos.dtype == query.dtype
+         and sin.dtype == query.dtype and cos.stride(1) == 1 and cos.stride() == sin.stride(),
+         f"cos/sin must be [P, {d}] tables of {query.dtype} with equal strides")
+    if positions is not None:
+        _req(positions.dtype == torch.int64 and positions.numel() == T and positions.is_contiguous(),
+             "positions must be contiguous int64 [T]")
+        _dev(positions, query, "positions")
+    else:
+        _req(cos.shape[0] >= T, "without positions the tables need one row per token")
+    _req(slot_mapping.dtype == torch.int64 and slot_mapping.numel() == T and slot_mapping.is_contiguous(),
+         "slot_mapping must be contiguous int64 [T]")
+    for t, n in ((key, "key"), (value, "value"), (out, "query_out"), (cos, "cos"), (sin, "sin"),
+                 (k_pool, "k_pool"), (slot_mapping, "slot_mapping")):
+        _dev(t, query, n)
+    _req(k_pool.dtype in (query.dtype, torch.float8_e4m3fn),
+         f"pool dtype {k_pool.dtype} must be {query.dtype} or float8_e4m3fn")
+    ks, vs = _check_scales(k_scale, v_scale, k_pool, hkv)
+    if T == 0:
+        return out
+    rc = lib.aicomp_rope_kv_append(
+        query.data_ptr(), out.data_ptr(), query.stride(0), query.stride(1), out.stride(0), out.stride(1),
+        key.data_ptr(), value.data_ptr(), key.stride(0), key.stride(1), cos.data_ptr(), sin.data_ptr(),
+        cos.stride(0), cos.shape[0], _ptr(positions), k_pool.data_ptr(), v_pool.data_ptr(),
+        slot_mapping.data_ptr(), T, hq, hkv, d, bs, nb, _dt(query, "query"), _dt(k_pool, "pool"),
+        _ptr(ks), _ptr(vs), _stream(query))
+    _lib.check(rc, lib)
+    return out

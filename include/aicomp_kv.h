@@ -174,6 +174,44 @@ int aicomp_paged_prefill_attn(void* out, const void* query,
                               const float* k_scale, const float* v_scale,
                               void* stream);
 
+/*
+ * Rotary position embedding of Q and K fused with the KV append: one launch for
+ *   q_embed = (q * cos) + (rotate_half(q) * sin)
+ *   k_embed = (k * cos) + (rotate_half(k) * sin)   (compiler_fx/modeling_llama.py:200-231,
+ *                                                   call site :582)
+ * and the append of k_embed / value                (kv_cache.py:387-388), with the KV heads
+ * stored once instead of repeat_kv's G copies      (modeling_llama.py:268-277, :589-590).
+ *
+ *   q_in, q_out     [T, Hq, D] of in_dtype (F32 or BF16); element (t,h,d) at
+ *                   t*token_stride + h*head_stride + d of the respective stride pair;
+ *                   q_out may be q_in (in place)
+ *   key, value      [T, Hkv, D] of in_dtype, strides as in aicomp_kv_append (the three inputs
+ *                   may be slices of one fused QKV projection output)
+ *   cos, sin        tables of in_dtype, row r at r*table_stride, D columns each (the
+ *                   reference's cos/sin, cast to the tensor type: modeling_llama.py:150-168)
+ *   positions       [T] int64 table row of each token, or NULL: token t uses row t (the
+ *                   per-call cos/sin the reference passes as position_embeddings)
+ *   table_rows      rows in the tables; a token whose position is outside is left alone
+ *   slot_mapping    [T] int64 as in aicomp_kv_append (slot < 0: Q is still rotated, K/V of
+ *                   that token are not stored)
+ *   pool_dtype      in_dtype (K rotated, V copied raw) or FP8_E4M3 (both quantised like
+ *                   aicomp_kv_append, K after the rotation)
+ * Every product and the sum are rounded to in_dtype one after the other, without fused
+ * multiply-add: bit-identical to the reference's eager evaluation.  D % 16 == 0; pointers
+ * and strides 16-byte aligned.
+ */
+int aicomp_rope_kv_append(const void* q_in, void* q_out,
+                          int64_t q_token_stride, int64_t q_head_stride,
+                          int64_t qo_token_stride, int64_t qo_head_stride,
+                          const void* key, const void* value,
+                          int64_t kv_token_stride, int64_t kv_head_stride,
+                          const void* cos, const void* sin, int64_t table_stride,
+                          int64_t table_rows, const int64_t* positions,
+                          void* k_pool, void* v_pool, const int64_t* slot_mapping,
+                          int64_t num_tokens, int num_q_heads, int num_kv_heads, int head_dim,
+                          int block_size, int64_t num_blocks, int in_dtype, int pool_dtype,
+                          const float* k_scale, const float* v_scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
