@@ -118,12 +118,14 @@ class StepPlan:
     context_lens: torch.Tensor            # [S] int32, after this step's append
     cu_q_lens: torch.Tensor               # [S+1] int32
     slot_mapping: torch.Tensor            # [T] int64
+    positions: torch.Tensor               # [T] int64 position of each new token in its sequence
     preempted: List[object]               # sequences sent back to the waiting queue by this call
     # host copies of the same arrays (what the tests and the oracle read)
     host_block_table: np.ndarray = None
     host_context_lens: np.ndarray = None
     host_cu_q_lens: np.ndarray = None
     host_slot_mapping: np.ndarray = None
+    host_positions: np.ndarray = None
 
     @property
     def num_seqs(self) -> int:
@@ -222,8 +224,9 @@ class StepPlanner:
         self._maxnew = np.zeros(max_seqs, dtype=np.int64)     # -1: unbounded
         self._arr = np.zeros(max_seqs, dtype=np.int64)
         self._live = np.zeros(max_seqs, dtype=bool)
-        # packed layout (bytes): slot_mapping int64 [T] | block_table int32 [S*MB] | context_lens [S] | cu_q_lens [S+1]
-        cap = 8 * max_num_batched_tokens + 4 * (max_seqs * MB + 2 * max_seqs + 1) + 64
+        # packed layout (bytes): slot_mapping int64 [T] | positions int64 [T] | block_table int32 [S*MB] |
+        # context_lens [S] | cu_q_lens [S+1]
+        cap = 16 * max_num_batched_tokens + 4 * (max_seqs * MB + 2 * max_seqs + 1) + 64
         self._staging = _Staging(cap, self.device, staging_depth)
 
     # ------------------------------------------------------------------ requests
@@ -315,7 +318,10 @@ class StepPlanner:
             self._nblk[r] += need
         return True
 
-    def schedule(self) -> Optional[StepPlan]:
+    def schedule(self, decode: Optional[Iterable[object]] = None) -> Optional[StepPlan]:
+        """Plan one step.  ``decode`` restricts which running sequences may take their one
+        token this step (default: all of them); a driver that ingests a whole batch of prompts
+        before its first decode step passes ``()`` until the last prompt is in."""
         budget = self.max_num_batched_tokens
         BS = self.block_size
         preempted: List[object] = []
@@ -324,6 +330,11 @@ class StepPlanner:
         # 1. one token for every running sequence past its prompt, oldest first (vectorised)
         dec = np.flatnonzero(self._live & (self._len >= self._prompt) &
                              ((self._maxnew < 0) | (self._len - self._orig + 1 < self._maxnew)))
+        if decode is not None:
+            allowed = np.zeros(self.max_seqs, dtype=bool)
+            rows = [self._row_of[sid] for sid in decode if sid in self._row_of]
+            allowed[rows] = True
+            dec = dec[allowed[dec]]
         if dec.size:
             dec = dec[np.argsort(self._arr[dec], kind="stable")][:budget]
             if int(self._len[dec].max()) + 1 > self.max_seq_len:
@@ -410,11 +421,13 @@ class StepPlanner:
         T = int(new_lens.sum())
         i = self._staging.next()
         raw = self._staging.host[i].numpy()
-        off_bt = 8 * T
+        off_pos = 8 * T
+        off_bt = 16 * T
         off_cl = off_bt + 4 * S * MB
         off_cu = off_cl + 4 * S
         end = off_cu + 4 * (S + 1)
-        slot = raw[:off_bt].view(np.int64)
+        slot = raw[:off_pos].view(np.int64)
+        posn = raw[off_pos:off_bt].view(np.int64)
         bt = raw[off_bt:off_cl].view(np.int32).reshape(S, MB)
         cl = raw[off_cl:off_cu].view(np.int32)
         cu = raw[off_cu:end].view(np.int32)
@@ -425,9 +438,11 @@ class StepPlanner:
         for k in range(npre):                                   # prompt chunks: a few per step
             pos = np.arange(start[k], start[k] + new_lens[k])
             slot[cu[k]:cu[k + 1]] = bt[k, pos // BS].astype(np.int64) * BS + pos % BS
+            posn[cu[k]:cu[k + 1]] = pos
         if S > npre:                                            # one-token rows, all at once
             p1 = start[npre:].astype(np.int64)
             slot[cu[npre]:] = bt[np.arange(npre, S), p1 // BS].astype(np.int64) * BS + p1 % BS
+            posn[cu[npre]:] = p1
         np.add(start, new_lens, out=cl)
         self._len[rows] = cl
         d = self._staging.upload(i, end)
@@ -438,10 +453,11 @@ class StepPlanner:
             block_table=dv[off_bt:off_cl].view(torch.int32).view(S, MB),
             context_lens=dv[off_cl:off_cu].view(torch.int32),
             cu_q_lens=dv[off_cu:end].view(torch.int32),
-            slot_mapping=dv[:off_bt].view(torch.int64),
+            slot_mapping=dv[:off_pos].view(torch.int64),
+            positions=dv[off_pos:off_bt].view(torch.int64),
             preempted=preempted,
             host_block_table=bt.copy(), host_context_lens=cl.copy(), host_cu_q_lens=cu.copy(),
-            host_slot_mapping=slot.copy(),
+            host_slot_mapping=slot.copy(), host_positions=posn.copy(),
         )
 
 

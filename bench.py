@@ -182,7 +182,7 @@ def planner_bench(dev):
     host = (time.perf_counter() - t0) / n
     torch.cuda.synchronize()
     return {"decode_plan_host_us": host * 1e6, "seqs": plan.num_seqs,
-            "h2d_bytes_per_plan": int(8 * plan.total_new_tokens + 4 * (plan.block_table.numel() + 2 * plan.num_seqs + 1)),
+            "h2d_bytes_per_plan": int(16 * plan.total_new_tokens + 4 * (plan.block_table.numel() + 2 * plan.num_seqs + 1)),
             "note": "StepPlanner.schedule() per decode step, including the enqueue of its one H2D copy"}
 
 

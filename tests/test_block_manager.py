@@ -121,6 +121,7 @@ class Sim:
             for i in range(n):                       # brute-force slot formula
                 t = len(h) + i
                 assert sm[cu[r] + i] == O.slot_of(plan.host_block_table[r], t, BS)
+                assert plan.host_positions[cu[r] + i] == t
             h.extend(k[cu[r]:cu[r] + n, 0, 0].tolist())
             L = len(h)
             assert p.context_len(sid) == L
@@ -139,6 +140,7 @@ class Sim:
         assert (plan.context_lens.numpy() == plan.host_context_lens).all()
         assert (plan.cu_q_lens.numpy() == plan.host_cu_q_lens).all()
         assert (plan.slot_mapping.numpy() == plan.host_slot_mapping).all()
+        assert (plan.positions.numpy() == plan.host_positions).all()
         # pool accounting over every running sequence
         used = set()
         for sid in list(p._row_of):
