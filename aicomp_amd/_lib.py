@@ -22,6 +22,7 @@ SYMBOLS = (
     "aicomp_paged_decode_partition_size",
     "aicomp_paged_prefill_attn",
     "aicomp_rope_kv_append",
+    "aicomp_sample_tokens",
 )
 
 F32, BF16, FP8_E4M3 = 0, 1, 2
@@ -61,6 +62,8 @@ def _declare(lib: C.CDLL) -> None:
     lib.aicomp_rope_kv_append.restype = i32
     lib.aicomp_rope_kv_append.argtypes = [vp, vp, i64, i64, i64, i64, vp, vp, i64, i64, vp, vp, i64, i64, vp,
                                           vp, vp, vp, i64, i32, i32, i32, i32, i64, i32, i32, vp, vp, vp]
+    lib.aicomp_sample_tokens.restype = i32
+    lib.aicomp_sample_tokens.argtypes = [vp, vp, i64, vp, vp, i32, i32, f32, i32, f32, i32, i32, vp]
 
 
 def load() -> C.CDLL:

@@ -132,6 +132,26 @@ int aicomp_rope_kv_append(const void* q_in, void* q_out, int64_t q_token_stride,
                                  in_dtype, pool_dtype, k_scale, v_scale, (hipStream_t)stream);
 }
 
+int aicomp_sample_tokens(int64_t* out, const void* logits, int64_t row_stride, float* probs_out,
+                         const float* uniforms, int batch, int vocab, float temperature, int top_k,
+                         float top_p, int greedy, int logits_dtype, void* stream) {
+    AICOMP_REQUIRE(batch >= 0, AICOMP_KV_EINVAL, "sample_tokens: negative batch");
+    if (batch == 0) return AICOMP_KV_OK;
+    AICOMP_REQUIRE(out && logits, AICOMP_KV_EINVAL, "sample_tokens: null pointer");
+    AICOMP_REQUIRE(vocab > 0 && row_stride >= vocab, AICOMP_KV_EINVAL,
+                   "sample_tokens: bad sizes (vocab %d, row stride %lld)", vocab, (long long)row_stride);
+    AICOMP_REQUIRE(logits_dtype == AICOMP_KV_F32 || logits_dtype == AICOMP_KV_BF16, AICOMP_KV_EUNSUPPORTED,
+                   "sample_tokens: logits must be float32 or bfloat16 (got %d)", logits_dtype);
+    if (!greedy) {
+        AICOMP_REQUIRE(uniforms, AICOMP_KV_EINVAL, "sample_tokens: sampling needs uniforms");
+        AICOMP_REQUIRE(temperature > 0.f, AICOMP_KV_EINVAL,
+                       "sample_tokens: temperature must be positive (got %g)", (double)temperature);
+        AICOMP_REQUIRE(top_p == top_p, AICOMP_KV_EINVAL, "sample_tokens: top_p is NaN");
+    }
+    return launch_sample(out, logits, row_stride, probs_out, uniforms, batch, vocab, temperature, top_k,
+                         top_p, greedy ? 1 : 0, logits_dtype, (hipStream_t)stream);
+}
+
 int aicomp_paged_decode_partition_size(int batch, int num_q_heads, int num_kv_heads, int head_dim,
                                        int block_size, int max_blocks_per_seq, int q_dtype,
                                        int kv_dtype) {

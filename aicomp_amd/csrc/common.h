@@ -171,6 +171,9 @@ int launch_kv_append_last(const void* key, const void* value, int64_t token_stri
                           int pool_dtype, const float* k_scale, const float* v_scale,
                           hipStream_t stream);
 int launch_split_reduce(const DecodeArgs& a);
+int launch_sample(int64_t* out, const void* logits, int64_t row_stride, float* probs_out,
+                  const float* uniforms, int batch, int vocab, float temperature, int top_k, float top_p,
+                  int greedy, int dtype, hipStream_t stream);
 int launch_rope_kv_append(const void* q_in, void* q_out, int64_t q_ts, int64_t q_hs, int64_t qo_ts,
                           int64_t qo_hs, const void* key, const void* value, int64_t kv_ts,
                           int64_t kv_hs, const void* cos_tab, const void* sin_tab, int64_t tab_stride,

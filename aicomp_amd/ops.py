@@ -295,3 +295,35 @@ def rope_kv_append(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, 
         _ptr(ks), _ptr(vs), _stream(query))
     _lib.check(rc, lib)
     return out
+
+
+def sample_tokens(logits: torch.Tensor, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0,
+                  do_sample: bool = True, uniforms: Optional[torch.Tensor] = None,
+                  generator: Optional[torch.Generator] = None, return_probs: bool = False):
+    """Next token of every row of ``logits [B, V]`` (float32 or bfloat16), as ``_sample_token`` of the
+    reference picks it (opt_prime/opt_prime/inference.py:786-843): greedy argmax when ``do_sample``
+    is false, otherwise temperature, top-k, top-p and one draw per row.  ``logits`` is not modified.
+
+    ``uniforms [B]`` (float32 in [0, 1)) makes the draw reproducible; by default they come from
+    ``torch.rand`` with ``generator``.  Returns ``tokens [B]`` int64, or ``(tokens, probs [B, V])``.
+    """
+    lib = _lib.load()
+    _req(logits.is_cuda, "tensors must live on a ROCm device (there is no CPU path)")
+    _req(logits.dim() == 2 and logits.stride(1) == 1, "logits must be [B, V] with contiguous rows")
+    _req(logits.dtype in (torch.float32, torch.bfloat16), f"unsupported logits dtype {logits.dtype}")
+    B, V = logits.shape
+    out = torch.empty(B, dtype=torch.int64, device=logits.device)
+    probs = torch.empty(B, V, dtype=torch.float32, device=logits.device) if return_probs else None
+    if do_sample:
+        if uniforms is None:
+            uniforms = torch.rand(B, dtype=torch.float32, device=logits.device, generator=generator)
+        _req(uniforms.dtype == torch.float32 and uniforms.numel() == B and uniforms.is_contiguous(),
+             "uniforms must be contiguous float32 [B]")
+        _dev(uniforms, logits, "uniforms")
+    if B:
+        rc = lib.aicomp_sample_tokens(out.data_ptr(), logits.data_ptr(), logits.stride(0), _ptr(probs),
+                                      _ptr(uniforms) if do_sample else None, B, V, float(temperature),
+                                      int(top_k), float(top_p), 0 if do_sample else 1, _dt(logits, "logits"),
+                                      _stream(logits))
+        _lib.check(rc, lib)
+    return (out, probs) if return_probs else out

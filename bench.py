@@ -186,6 +186,49 @@ def planner_bench(dev):
             "note": "StepPlanner.schedule() per decode step, including the enqueue of its one H2D copy"}
 
 
+def sampler_bench(dev, batch=64, vocab=128256, temperature=0.8, top_k=50, top_p=0.9, reps=20):
+    """The step after the attention path: one token per row of [64, 128256] fp32 logits with
+    temperature / top-k / top-p (opt_prime/opt_prime/inference.py:786-843).  Beside the kernel, the
+    reference's own statement sequence run by torch on the same GPU (sort, cumsum, softmax, scatter,
+    multinomial) as the figure it replaces."""
+    import torch
+    from aicomp_amd import ops
+    g = torch.Generator(device=dev).manual_seed(0)
+    logits = torch.randn(batch, vocab, device=dev, generator=g) * 2.5
+    u = torch.rand(batch, device=dev, generator=g)
+
+    def ours():
+        return ops.sample_tokens(logits, temperature, top_k, top_p, uniforms=u)
+
+    def eager():
+        x = logits.clone() / temperature
+        k = min(top_k, x.size(-1))
+        x[x < torch.topk(x, k)[0][..., -1, None]] = float("-inf")
+        sl, si = torch.sort(x, descending=True)
+        cp = torch.cumsum(torch.softmax(sl, dim=-1), dim=-1)
+        rm = cp > top_p
+        rm[..., 1:] = rm[..., :-1].clone()
+        rm[..., 0] = 0
+        x[rm.scatter(-1, si, rm)] = float("-inf")
+        return torch.multinomial(torch.softmax(x, dim=-1), num_samples=1).squeeze(-1)
+
+    res = {}
+    for name, fn in (("kernel_us", ours), ("torch_eager_us", eager)):
+        for _ in range(3):
+            fn()
+        e0, e1 = _events(2)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        res[name] = e0.elapsed_time(e1) / reps * 1e3
+    res.update({"batch": batch, "vocab": vocab, "temperature": temperature, "top_k": top_k, "top_p": top_p,
+                "dtype": "f32", "logit_bytes": batch * vocab * 4})
+    return res
+
+
 def device_info():
     import torch
     p = torch.cuda.get_device_properties(0)
@@ -231,6 +274,15 @@ def profile_target(which, steps, warmup, dev):
             dst.copy_(src)
         torch.cuda.synchronize()
         print(f"copy: {steps + warmup} launches of {src.numel()} bytes read + {dst.numel()} bytes written")
+        return
+    if which == "sample":
+        g = torch.Generator(device=dev).manual_seed(0)
+        logits = torch.randn(64, 128256, device=dev, generator=g) * 2.5
+        u = torch.rand(64, device=dev, generator=g)
+        for _ in range(warmup + steps):
+            ops.sample_tokens(logits, 0.8, 50, 0.9, uniforms=u)
+        torch.cuda.synchronize()
+        print(f"sample: {steps + warmup} launches over [64, 128256] fp32 logits, temperature 0.8, top-k 50, top-p 0.9")
         return
     name = {"decode": "llama3_8b_decode", "append": "chunked_prefill_mixed", "prefill": "chunked_prefill_mixed",
             "decode_fp8": "llama3_70b_decode_fp8", "decode_long": "long_context_skewed",
@@ -322,7 +374,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
-    ap.add_argument("--only", choices=["decode", "append", "copy", "prefill", "decode_fp8", "decode_long", "rope"],
+    ap.add_argument("--only", choices=["decode", "append", "copy", "prefill", "decode_fp8", "decode_long", "rope", "sample"],
                     help="profiling target: launch just this kernel --steps times (no JSON line)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -370,6 +422,7 @@ def main():
                         "note": "decode call timed right after 1 GiB of unrelated writes"},
         "device": device_info(),
         "step_planner": planner_bench(dev),
+        "sampler": sampler_bench(dev),
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(w)

@@ -212,6 +212,30 @@ int aicomp_rope_kv_append(const void* q_in, void* q_out,
                           int block_size, int64_t num_blocks, int in_dtype, int pool_dtype,
                           const float* k_scale, const float* v_scale, void* stream);
 
+/*
+ * Token sampling, one launch per batch of rows.  Replaces _sample_token
+ * (opt_prime/opt_prime/inference.py:786-843): greedy argmax (:806-808), or
+ * logits / temperature (:811-812), top-k (:815-818: entries below the k-th largest value are
+ * removed, ties at that value stay), top-p (:821-837: in descending order an entry stays while
+ * the mass before it is <= top_p; the first always stays; mass = softmax of what top-k left),
+ * then a draw from the softmax of what is left (:840-841).
+ *
+ *   out           [B] int64 token ids
+ *   logits        [B, V] F32 or BF16, row b at b*row_stride elements; not modified
+ *   uniforms      [B] float in [0, 1): the draw is the inverse CDF in index order at
+ *                 uniforms[b] (the reference draws with torch.multinomial; the distribution is
+ *                 the same, the random stream is the caller's).  Not read when greedy.
+ *   probs_out     optional [B, V] float: the distribution the draw is made from
+ *   temperature   > 0 (ignored when greedy);  top_k <= 0 or >= V: off;  top_p >= 1: off
+ *   greedy        non-zero: argmax, lowest index among equal maxima
+ * Ties at the nucleus threshold are kept in index order.  Probability mass is summed exactly
+ * in 2^-40 fixed point, so a call is reproducible bit for bit.
+ */
+int aicomp_sample_tokens(int64_t* out, const void* logits, int64_t row_stride,
+                         float* probs_out, const float* uniforms,
+                         int batch, int vocab, float temperature, int top_k, float top_p,
+                         int greedy, int logits_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
