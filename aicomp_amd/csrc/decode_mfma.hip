@@ -701,15 +701,18 @@ streamk_decode_kernel(StreamKParams p) {
 // group).  The row's partials sit in consecutive slots first+row .. last+row (first / last
 // wave recorded by the main kernel); their weights 2^(m_i - M) are computed once (one lane
 // per partial) and parked in LDS, then each lane accumulates two output dims with
-// independent loads.  A single wave: reductions are shuffles, no barrier.
-__global__ void __launch_bounds__(64)
+// independent loads.  One wave per head: reductions are shuffles, no barrier.
+constexpr int RED_WGT = 256;       // weights parked in LDS per head; rows with more partials recompute the rest
+__global__ void __launch_bounds__(1024)
 streamk_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws_acc,
                       const float* __restrict__ ws_ml, const int* __restrict__ ws_rows,
                       const int32_t* __restrict__ context_lens, int hq, int hkv, int group,
                       const float* __restrict__ v_scale) {
-    const int kvh = blockIdx.x, seq = blockIdx.y, h = blockIdx.z;
-    const int lane = threadIdx.x;
-    __shared__ float wgt[SK_MAX_WAVES / 4];
+    // one workgroup per (KV head, sequence), one wave per head of the group
+    const int kvh = blockIdx.x, seq = blockIdx.y, h = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    __shared__ float wgt_all[16][RED_WGT];
+    float* wgt = wgt_all[h];
     const int64_t row = (int64_t)seq * hkv + kvh;
     bf16_t* o = out + ((int64_t)seq * hq + kvh * group + h) * D;
     if (context_lens[seq] <= 0) {            // no tiles, no partials: the output row is zero
@@ -728,21 +731,31 @@ streamk_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws_acc
     for (int i = lane; i < np; i += 64) {
         const float2 v = *(const float2*)(ml + (int64_t)i * group * 2);
         const float f = exp2f(v.x - mx);
-        wgt[i] = f;
+        if (i < RED_WGT) wgt[i] = f;
         den = fmaf(f, v.y, den);
     }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) den += __shfl_xor(den, off);
     const int64_t stride = (int64_t)group * D;
+    // eight partials (sixteen loads) in flight per step: a long row has tens of partials and
+    // the loop is pure load latency
     float n0 = 0.f, n1 = 0.f;
-    int i = 0;
-    for (; i + 2 <= np; i += 2) {
-        const float a0 = acc[i * stride], b0 = acc[i * stride + 64];
-        const float a1 = acc[(i + 1) * stride], b1 = acc[(i + 1) * stride + 64];
-        n0 = fmaf(wgt[i], a0, n0); n1 = fmaf(wgt[i], b0, n1);
-        n0 = fmaf(wgt[i + 1], a1, n0); n1 = fmaf(wgt[i + 1], b1, n1);
+    for (int i0 = 0; i0 < np; i0 += 8) {
+        float a[8], b[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = min(i0 + u, np - 1);
+            a[u] = acc[i * stride];
+            b[u] = acc[i * stride + 64];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = i0 + u;
+            const float f = i >= np ? 0.f : (i < RED_WGT ? wgt[i] : exp2f(ml[(int64_t)i * group * 2] - mx));
+            n0 = fmaf(f, a[u], n0);
+            n1 = fmaf(f, b[u], n1);
+        }
     }
-    if (i < np) { n0 = fmaf(wgt[i], acc[i * stride], n0); n1 = fmaf(wgt[i], acc[i * stride + 64], n1); }
     const float inv = den > 0.f ? (v_scale ? v_scale[kvh] : 1.f) / den : 0.f;
     o[lane].bits = f32_to_bf16(n0 * inv);
     o[lane + 64].bits = f32_to_bf16(n1 * inv);
@@ -803,7 +816,7 @@ int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
     else
         hipLaunchKernelGGL(streamk_decode_kernel<false>, dim3(wgs), dim3(256), 0, a.stream, p);
     AICOMP_HIP_LAUNCH_CHECK();
-    hipLaunchKernelGGL(streamk_reduce_kernel, dim3(a.hkv, (unsigned)a.rows, group), dim3(64), 0, a.stream,
+    hipLaunchKernelGGL(streamk_reduce_kernel, dim3(a.hkv, (unsigned)a.rows), dim3(64 * group), 0, a.stream,
                        (bf16_t*)a.out, p.ws_acc, p.ws_ml, p.ws_rows, a.context_lens, a.hq, a.hkv, group,
                        a.v_scale);
     AICOMP_HIP_LAUNCH_CHECK();
