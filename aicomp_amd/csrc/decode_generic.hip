@@ -35,22 +35,21 @@ __device__ __forceinline__ uint2 stream_ld8(const void* p) {
 template <typename KV_T> struct KvLoad;
 template <> struct KvLoad<float> {
     static constexpr int N = 4;
-    __device__ __forceinline__ static void load(const float* p, float* f) {
-        uint4 r = stream_ld16(p);
-        Vec16<float>::unpack(r, f);
-    }
+    typedef uint4 Raw;
+    __device__ __forceinline__ static Raw raw(const float* p) { return stream_ld16(p); }
+    __device__ __forceinline__ static void unpack(const Raw& r, float* f) { Vec16<float>::unpack(r, f); }
 };
 template <> struct KvLoad<bf16_t> {
     static constexpr int N = 8;
-    __device__ __forceinline__ static void load(const bf16_t* p, float* f) {
-        uint4 r = stream_ld16(p);
-        Vec16<bf16_t>::unpack(r, f);
-    }
+    typedef uint4 Raw;
+    __device__ __forceinline__ static Raw raw(const bf16_t* p) { return stream_ld16(p); }
+    __device__ __forceinline__ static void unpack(const Raw& r, float* f) { Vec16<bf16_t>::unpack(r, f); }
 };
 template <> struct KvLoad<fp8_t> {
     static constexpr int N = 8;
-    __device__ __forceinline__ static void load(const fp8_t* p, float* f) {
-        uint2 r = stream_ld8(p);
+    typedef uint2 Raw;
+    __device__ __forceinline__ static Raw raw(const fp8_t* p) { return stream_ld8(p); }
+    __device__ __forceinline__ static void unpack(const Raw& r, float* f) {
         const uint32_t w[2] = {r.x, r.y};
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -161,38 +160,62 @@ paged_attn_generic_kernel(GenericParams p) {
     const int32_t* table = p.block_table + (int64_t)seq * p.block_table_stride;
     const KV_T* kp = (const KV_T*)p.k_pool;
     const KV_T* vp = (const KV_T*)p.v_pool;
-    const int steps = (end - start + NW * TPW - 1) / (NW * TPW);
-
-    for (int it = 0; it < steps; ++it) {
-        const int tok = start + it * NW * TPW + w * TPW + sub;
-        const bool valid = tok < end;
-        float kf[N], vf[N];
-        int64_t base = 0;
-        if (valid) {
+    // Two tokens per lane group and step, and the next step's four K/V chunks are requested before
+    // the current ones are used: eight 16-byte loads in flight per lane.  One running-max update
+    // (one rescale of the accumulators) serves both tokens.
+    constexpr int STEP = 2 * NW * TPW;                 // tokens per workgroup step
+    const int steps = (end - start + STEP - 1) / STEP;
+    typedef typename KvLoad<KV_T>::Raw Raw;
+    auto fetch = [&](int it, Raw (&kraw)[2], Raw (&vraw)[2]) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int tok = min(start + it * STEP + u * NW * TPW + w * TPW + sub, end - 1);   // clamped: always loadable
             int64_t blk = table[tok / p.bs];
             blk = blk < 0 ? 0 : (blk >= p.num_blocks ? p.num_blocks - 1 : blk);  // never leave the pool
-            base = ((blk * p.hkv + kvh) * p.bs + tok % p.bs) * D + lr * N;
-            KvLoad<KV_T>::load(kp + base, kf);
-            KvLoad<KV_T>::load(vp + base, vf);
-        } else {
+            const int64_t base = ((blk * p.hkv + kvh) * p.bs + tok % p.bs) * D + lr * N;
+            kraw[u] = KvLoad<KV_T>::raw(kp + base);
+            vraw[u] = KvLoad<KV_T>::raw(vp + base);
+        }
+    };
+    Raw kcur[2], vcur[2], knext[2], vnext[2];
+    fetch(0, kcur, vcur);
+    for (int it = 0; it < steps; ++it) {
+        if (it + 1 < steps) fetch(it + 1, knext, vnext);
+        const int tok0 = start + it * STEP + w * TPW + sub;
+        const bool valid0 = tok0 < end, valid1 = tok0 + NW * TPW < end;
+        float k0[N], v0[N], k1[N], v1[N];
+        KvLoad<KV_T>::unpack(kcur[0], k0);
+        KvLoad<KV_T>::unpack(kcur[1], k1);
+        KvLoad<KV_T>::unpack(vcur[0], v0);
+        KvLoad<KV_T>::unpack(vcur[1], v1);
+        if (!valid0) {
 #pragma unroll
-            for (int e = 0; e < N; ++e) { kf[e] = 0.f; vf[e] = 0.f; }
+            for (int e = 0; e < N; ++e) v0[e] = 0.f;           // a clamped reload may hold anything
+        }
+        if (!valid1) {
+#pragma unroll
+            for (int e = 0; e < N; ++e) v1[e] = 0.f;
         }
 #pragma unroll
         for (int g = 0; g < GMAX; ++g) {
-            float s = 0.f;
+            float s0 = 0.f, s1 = 0.f;
 #pragma unroll
-            for (int e = 0; e < N; ++e) s = fmaf(q[g][e], kf[e], s);
+            for (int e = 0; e < N; ++e) { s0 = fmaf(q[g][e], k0[e], s0); s1 = fmaf(q[g][e], k1[e], s1); }
 #pragma unroll
-            for (int o = 1; o < LPR; o <<= 1) s += __shfl_xor(s, o);
-            const float m_new = valid ? fmaxf(m[g], s) : m[g];
-            const float alpha = exp2f(m[g] - m_new);
-            const float pr = valid ? exp2f(s - m_new) : 0.f;
+            for (int o = 1; o < LPR; o <<= 1) { s0 += __shfl_xor(s0, o); s1 += __shfl_xor(s1, o); }
+            float m_new = m[g];
+            if (valid0) m_new = fmaxf(m_new, s0);
+            if (valid1) m_new = fmaxf(m_new, s1);
+            const float alpha = __builtin_amdgcn_exp2f(m[g] - m_new);
+            const float p0 = valid0 ? __builtin_amdgcn_exp2f(s0 - m_new) : 0.f;
+            const float p1 = valid1 ? __builtin_amdgcn_exp2f(s1 - m_new) : 0.f;
             m[g] = m_new;
-            l[g] = l[g] * alpha + pr;
+            l[g] = l[g] * alpha + p0 + p1;
 #pragma unroll
-            for (int e = 0; e < N; ++e) acc[g][e] = fmaf(pr, vf[e], acc[g][e] * alpha);
+            for (int e = 0; e < N; ++e) acc[g][e] = fmaf(p1, v1[e], fmaf(p0, v0[e], acc[g][e] * alpha));
         }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) { kcur[u] = knext[u]; vcur[u] = vnext[u]; }
     }
 
     // merge the TPW lane groups of the wave

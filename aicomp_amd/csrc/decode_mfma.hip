@@ -6,8 +6,12 @@
 // K and V are read once, in place, through the block table.
 //
 // Shape covered: head_dim 128, block_size 16, bf16 queries, bf16 or fp8-e4m3
-// pools, up to 16 query heads per KV head.  Everything else goes to the
-// vector-ALU kernel.
+// pools, up to 16 query heads per KV head; and head_dim 64 (up to 8 heads per KV
+// head) by treating two consecutive tokens, which are contiguous in the pool, as
+// one 128-element row: every head takes two B-operand columns, one per token
+// parity, with the query in the matching half of the row and zeros in the other,
+// and the two columns' partial softmaxes are merged at the end.  Same instruction
+// stream per byte as head_dim 128.  Everything else goes to the vector-ALU kernel.
 //
 // HBM-bound: per sequence 2 * L * Hkv * D * e_kv bytes of K/V are streamed and
 // used exactly once; 4 * G flop per byte (bf16), far below the MFMA roof, so
@@ -34,9 +38,7 @@
 // Softmax      log2 domain, running max per head made wave-uniform with two
 //              wave shuffles (lanes l, l^16, l^32, l^48 hold the same head).
 // Split-K      partitions write (max, sum, unnormalised output) to the
-//              workspace; the workgroup that finishes a (sequence, KV head)'s
-//              last partition (device-scope counter) merges them in the same
-//              launch, so a decode call is one kernel.
+//              workspace; a second, small kernel merges them.
 #include "common.h"
 
 namespace aicomp {
@@ -134,6 +136,30 @@ __device__ __forceinline__ void load_tile(TileRegs<FP8>& t, const void* pool, in
     }
 }
 
+// head_dim 64: a 32-row tile of 128-element rows is 64 tokens, each row a PAIR of consecutive
+// tokens (token 2r in elements 0..63, token 2r+1 in 64..127; contiguous in the pool).  Four
+// blocks of 8 such rows.
+template <bool FP8>
+__device__ __forceinline__ void load_tile_pair(TileRegs<FP8>& t, const void* pool, int64_t blk0, int64_t blk1,
+                                               int64_t blk2, int64_t blk3, int hkv, int kvh, int lane) {
+    const int64_t blk[4] = {blk0, blk1, blk2, blk3};
+    if constexpr (FP8) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const uint2* p = (const uint2*)pool + (blk[b] * hkv + kvh) * (BS * 64 / 8) + lane;
+            t.r[2 * b] = TILE_LD(p);
+            t.r[2 * b + 1] = TILE_LD(p + 64);
+        }
+    } else {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const uint4* p = (const uint4*)pool + (blk[b] * hkv + kvh) * (BS * 64 / 8) + lane;
+            t.r[2 * b] = TILE_LD(p);
+            t.r[2 * b + 1] = TILE_LD(p + 64);
+        }
+    }
+}
+
 template <bool FP8>
 __device__ __forceinline__ uint4 tile_bf16(const TileRegs<FP8>& t, int i) {
     if constexpr (FP8) return fp8x8_to_bf16x8(t.r[i]);
@@ -153,17 +179,28 @@ struct WaveState {
 // One 32-token tile: K registers -> LDS -> S^T = K Q^T -> online softmax -> O^T += V^T P^T.
 // NEXT: prefetch the wave's next tile (blocks nb0/nb1) into the same registers.
 // MASK: the tile crosses `end`; scores beyond it are dropped and their V rows zeroed.
-template <bool FP8, bool NEXT, bool MASK>
+// PAIR: rows are token pairs (head_dim 64): row r of the tile holds tokens tile_start + 2r and
+// + 2r + 1, the B-operand columns are (head, parity) pairs, column c scoring token 2r + (c & 1).
+template <bool FP8, bool NEXT, bool MASK, bool PAIR = false>
 __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, TileRegs<FP8>& vr,
                                              const bf16x8_t (&qf)[4], unsigned char* kt, int wr_off,
                                              int rd_off, const void* k_pool, const void* v_pool,
                                              int64_t nb0, int64_t nb1, int hkv, int kvh_next, int lane,
-                                             int g4, int tile_start, int end, float cmul) {
+                                             int g4, int tile_start, int end, float cmul,
+                                             int64_t nb2 = 0, int64_t nb3 = 0) {
     // ---- K tile -> LDS, then prefetch the next K tile into the same registers
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-        *(uint4*)(kt + wr_off + i * 4 * KROW) = tile_bf16<FP8>(kr, i);
-    if (NEXT) load_tile<FP8>(kr, k_pool, nb0, nb1, hkv, kvh_next, lane);
+    for (int i = 0; i < 8; ++i) {
+        uint4 kk = tile_bf16<FP8>(kr, i);
+        // PAIR: a row's two tokens share every dot product (the query column is zero over the other
+        // token's half), so a token beyond the context must not leave non-finite values in the row
+        if (PAIR && MASK && tile_start + 2 * (4 * i + g4) + ((lane & 15) >> 3) >= end) kk = make_uint4(0, 0, 0, 0);
+        *(uint4*)(kt + wr_off + i * 4 * KROW) = kk;
+    }
+    if (NEXT) {
+        if constexpr (PAIR) load_tile_pair<FP8>(kr, k_pool, nb0, nb1, nb2, nb3, hkv, kvh_next, lane);
+        else load_tile<FP8>(kr, k_pool, nb0, nb1, hkv, kvh_next, lane);
+    }
 
     // ---- S^T = K Q^T for the two 16-token sub-tiles
     f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
@@ -181,7 +218,8 @@ __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, T
     if (MASK) {
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
-            const int tok = tile_start + 16 * (k >> 2) + 4 * (k & 3) + g4;
+            const int r = 16 * (k >> 2) + 4 * (k & 3) + g4;
+            const int tok = PAIR ? tile_start + 2 * r + (lane & 1) : tile_start + r;
             if (tok >= end) sc[k] = NEG_BIG;
         }
     }
@@ -215,7 +253,9 @@ __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, T
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         vv[i] = tile_bf16<FP8>(vr, i);
-        if (MASK && tile_start + 4 * i + g4 >= end) vv[i] = make_uint4(0, 0, 0, 0);
+        // PAIR: chunks 8..15 of a row belong to the pair's second token
+        const int vtok = PAIR ? tile_start + 2 * (4 * i + g4) + ((lane & 15) >> 3) : tile_start + 4 * i + g4;
+        if (MASK && vtok >= end) vv[i] = make_uint4(0, 0, 0, 0);
     }
     uint4 af[8];
 #pragma unroll
@@ -227,17 +267,23 @@ __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, T
         af[j].z = __builtin_amdgcn_perm(v0[4 * 5 + (j >> 1)], v0[4 * 4 + (j >> 1)], sel);
         af[j].w = __builtin_amdgcn_perm(v0[4 * 7 + (j >> 1)], v0[4 * 6 + (j >> 1)], sel);
     }
-    if (NEXT) load_tile<FP8>(vr, v_pool, nb0, nb1, hkv, kvh_next, lane);
+    if (NEXT) {
+        if constexpr (PAIR) load_tile_pair<FP8>(vr, v_pool, nb0, nb1, nb2, nb3, hkv, kvh_next, lane);
+        else load_tile<FP8>(vr, v_pool, nb0, nb1, hkv, kvh_next, lane);
+    }
 #pragma unroll
     for (int j = 0; j < 8; ++j)
         st.O[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, af[j]), pf, st.O[j], 0, 0, 0);
 }
 
-template <bool FP8>
+template <bool FP8, bool PAIR>
 __global__ void __launch_bounds__(256, 2)
 paged_decode_mfma_kernel(MfmaParams p) {
     // KV head fastest: the workgroups launched together read the Hkv slices of the same
     // physical blocks, i.e. one contiguous Hkv*4 KB piece of each pool
+    constexpr int DQ = PAIR ? 64 : D;            // head_dim of the tensors
+    constexpr int TT = PAIR ? 2 * TILE : TILE;   // tokens per tile
+    constexpr int BPT = TT / BS;                 // blocks per tile
     const int kvh = blockIdx.x;
     const int part = blockIdx.y;
     const int seq = blockIdx.z;
@@ -247,6 +293,7 @@ paged_decode_mfma_kernel(MfmaParams p) {
     const int r16 = lane & 15;      // MFMA row / column index of this lane
     const int g4 = lane >> 4;       // MFMA k-group of this lane
     const int G = p.group;
+    const int ncol = PAIR ? 2 * G : G;           // B-operand columns in use
     const int start = part * p.partition_size;
     const int blk_base = start / BS;
 
@@ -259,14 +306,23 @@ paged_decode_mfma_kernel(MfmaParams p) {
     int tab = (blk_base + lane < p.max_blocks) ? table[blk_base + lane] : 0;
 
     // Q as the B operand of S^T = K Q^T: column = head r16, k-slots = dims 32s + 8*g4 ..
+    // PAIR: column c is (head c/2, parity c%2); a row of the K tile is [token 2r | token 2r+1], so
+    // the column carries the query in elements 0..63 (parity 0) or 64..127 (parity 1), zeros elsewhere.
     bf16x8_t qf[4];
     {
-        const uint4* qp = (const uint4*)((const bf16_t*)p.query +
-                                         ((int64_t)seq * p.hq + kvh * G + min(r16, G - 1)) * D + 8 * g4);
+        const int h = PAIR ? (r16 >> 1) : r16;
+        const bf16_t* qrow = (const bf16_t*)p.query + ((int64_t)seq * p.hq + kvh * G + min(h, G - 1)) * DQ;
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            uint4 v = qp[s * 4];
-            if (r16 >= G) v = make_uint4(0, 0, 0, 0);
+            const int e0 = 32 * s + 8 * g4;                       // first element of this k-slot in the row
+            bool use = r16 < ncol;
+            int src = e0;
+            if constexpr (PAIR) {
+                use = use && ((e0 >= 64) == ((r16 & 1) != 0));
+                src = e0 & 63;
+            }
+            uint4 v = *(const uint4*)(qrow + src);
+            if (!use) v = make_uint4(0, 0, 0, 0);
             qf[s] = __builtin_bit_cast(bf16x8_t, v);
         }
     }
@@ -274,13 +330,13 @@ paged_decode_mfma_kernel(MfmaParams p) {
     const int len = min(p.context_lens[seq], p.max_blocks * BS);   // never read past the table row
     if (start >= len) {
         if (len <= 0 && part == 0) {   // nothing to attend to: the output row is defined as zero
-            bf16_t* o = (bf16_t*)p.out + ((int64_t)seq * p.hq + kvh * G) * D;
-            for (int i = tid; i < G * D; i += blockDim.x) o[i].bits = 0;
+            bf16_t* o = (bf16_t*)p.out + ((int64_t)seq * p.hq + kvh * G) * DQ;
+            for (int i = tid; i < G * DQ; i += blockDim.x) o[i].bits = 0;
         }
         return;
     }
     const int end = min(len, start + p.partition_size);
-    const int ntiles = (end - start + TILE - 1) / TILE;
+    const int ntiles = (end - start + TT - 1) / TT;
 
     __shared__ __attribute__((aligned(16))) unsigned char lds[NWAVES * KTILE_BYTES];
     __shared__ float sm_m[NWAVES][16];
@@ -295,15 +351,17 @@ paged_decode_mfma_kernel(MfmaParams p) {
     for (int j = 0; j < 8; ++j) st.O[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     // physical blocks of tile tt (wave-uniform); the held table slice is refilled every 64 blocks
-    auto tile_blocks = [&](int tt, int64_t& b0, int64_t& b1) {
-        const int i0 = 2 * tt;
+    int64_t bb[4] = {0, 0, 0, 0};
+    auto tile_blocks = [&](int tt) {
+        const int i0 = BPT * tt;
         if (i0 - tab_first >= 64) {
             tab_first = i0;
             tab = (blk_base + i0 + lane < p.max_blocks) ? table[blk_base + i0 + lane] : 0;
             __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0) here, so the common path never waits on `tab`
         }
-        b0 = clamp_block(__builtin_amdgcn_readlane(tab, i0 - tab_first), p.num_blocks);
-        b1 = clamp_block(__builtin_amdgcn_readlane(tab, i0 + 1 - tab_first), p.num_blocks);
+#pragma unroll
+        for (int j = 0; j < BPT; ++j)
+            bb[j] = clamp_block(__builtin_amdgcn_readlane(tab, i0 + j - tab_first), p.num_blocks);
     };
 
     // LDS addresses: write row = 4i + lane/16, chunk lane%16;
@@ -313,36 +371,41 @@ paged_decode_mfma_kernel(MfmaParams p) {
 
     if (w < ntiles) {
         TileRegs<FP8> kr, vr;
-        int64_t b0, b1;
-        tile_blocks(w, b0, b1);
+        tile_blocks(w);
         // Q must have landed before the tile loads are issued: the loop's waits then count
         // only tile loads, so a wave computes on tile t while tile t+1 is still in flight.
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
-        load_tile<FP8>(kr, p.k_pool, b0, b1, p.hkv, kvh, lane);
-        load_tile<FP8>(vr, p.v_pool, b0, b1, p.hkv, kvh, lane);
+        if constexpr (PAIR) {
+            load_tile_pair<FP8>(kr, p.k_pool, bb[0], bb[1], bb[2], bb[3], p.hkv, kvh, lane);
+            load_tile_pair<FP8>(vr, p.v_pool, bb[0], bb[1], bb[2], bb[3], p.hkv, kvh, lane);
+        } else {
+            load_tile<FP8>(kr, p.k_pool, bb[0], bb[1], p.hkv, kvh, lane);
+            load_tile<FP8>(vr, p.v_pool, bb[0], bb[1], p.hkv, kvh, lane);
+        }
         int tt = w;
         for (; tt + NWAVES < ntiles; tt += NWAVES) {      // steady state: never the partition's last tile
-            tile_blocks(tt + NWAVES, b0, b1);
-            process_tile<FP8, true, false>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, b0,
-                                           b1, p.hkv, kvh, lane, g4, start + tt * TILE, end, cmul);
+            tile_blocks(tt + NWAVES);
+            process_tile<FP8, true, false, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, bb[0],
+                                                 bb[1], p.hkv, kvh, lane, g4, start + tt * TT, end, cmul,
+                                                 bb[2], bb[3]);
         }
-        const int tile_start = start + tt * TILE;
-        if (tile_start + TILE > end)
-            process_tile<FP8, false, true>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
-                                           p.hkv, kvh, lane, g4, tile_start, end, cmul);
+        const int tile_start = start + tt * TT;
+        if (tile_start + TT > end)
+            process_tile<FP8, false, true, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
+                                                 p.hkv, kvh, lane, g4, tile_start, end, cmul);
         else
-            process_tile<FP8, false, false>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
-                                            p.hkv, kvh, lane, g4, tile_start, end, cmul);
+            process_tile<FP8, false, false, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
+                                                  p.hkv, kvh, lane, g4, tile_start, end, cmul);
     }
     const float m = st.m;
     float lsum = st.lsum;
     f32x4_t (&O)[8] = st.O;
 
-    // ---- wave result: lane (head r16, g4) holds O^T[dim 32*g4 + 8*i + j][head] in O[j][i]
+    // ---- wave result: lane (column r16, g4) holds O^T[element 32*g4 + 8*i + j][column] in O[j][i]
     lsum += __shfl_xor(lsum, 16);
     lsum += __shfl_xor(lsum, 32);
-    float* osm = (float*)kt;        // this wave's own K tile region, G*128 floats <= 8704 bytes
-    if (r16 < G) {
+    float* osm = (float*)kt;        // this wave's own K tile region, 16 columns * 128 floats <= 8704 bytes
+    if (r16 < ncol) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             float4 a = make_float4(O[0][i], O[1][i], O[2][i], O[3][i]);
@@ -355,28 +418,36 @@ paged_decode_mfma_kernel(MfmaParams p) {
     }
     __syncthreads();
 
+    // merge of the waves (PAIR: and of the two parity columns of a head, whose useful halves are
+    // elements 0..63 and 64..127 of their accumulators)
     const float vs = FP8 ? p.v_scale[kvh] : 1.f;
-    const int nvalid = (len + p.partition_size - 1) / p.partition_size;   // partitions holding tokens
     const bool direct = p.num_parts == 1;     // unsplit call: no merge needed
-    for (int idx = tid; idx < G * D; idx += 256) {
-        const int h = idx >> 7, dd = idx & 127;
-        float mxw = sm_m[0][h];
+    constexpr int NPAR = PAIR ? 2 : 1;
+    for (int idx = tid; idx < G * DQ; idx += 256) {
+        const int h = idx / DQ, dd = idx % DQ;
+        float mxw = NEG_BIG;
 #pragma unroll
-        for (int ww = 1; ww < NWAVES; ++ww) mxw = fmaxf(mxw, sm_m[ww][h]);
+        for (int ww = 0; ww < NWAVES; ++ww)
+#pragma unroll
+            for (int par = 0; par < NPAR; ++par) mxw = fmaxf(mxw, sm_m[ww][NPAR * h + par]);
         float num = 0.f, den = 0.f;
 #pragma unroll
         for (int ww = 0; ww < NWAVES; ++ww) {
-            const float f = exp2f(sm_m[ww][h] - mxw);
-            num = fmaf(f, ((const float*)(lds + ww * KTILE_BYTES))[h * D + dd], num);
-            den = fmaf(f, sm_l[ww][h], den);
+#pragma unroll
+            for (int par = 0; par < NPAR; ++par) {
+                const int c = NPAR * h + par;
+                const float f = exp2f(sm_m[ww][c] - mxw);
+                num = fmaf(f, ((const float*)(lds + ww * KTILE_BYTES))[c * D + dd + 64 * par], num);
+                den = fmaf(f, sm_l[ww][c], den);
+            }
         }
         const int head = kvh * G + h;
         if (direct) {
-            ((bf16_t*)p.out)[((int64_t)seq * p.hq + head) * D + dd].bits =
+            ((bf16_t*)p.out)[((int64_t)seq * p.hq + head) * DQ + dd].bits =
                 f32_to_bf16(den > 0.f ? vs * num / den : 0.f);
         } else {
             const int64_t slot = ((int64_t)seq * p.hq + head) * p.num_parts + part;
-            p.ws_acc[slot * D + dd] = num;
+            p.ws_acc[slot * DQ + dd] = num;
             if (dd == 0) { p.ws_ml[slot * 2] = mxw; p.ws_ml[slot * 2 + 1] = den; }
         }
     }
@@ -763,17 +834,21 @@ streamk_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws_acc
 
 }  // namespace
 
+// head_dim 128, or head_dim 64 handled as rows of token pairs (two B-operand columns per head,
+// hence groups up to 8 and partitions of whole 64-token tiles)
 bool decode_mfma_supported(const DecodeArgs& a) {
     const int group = a.hkv > 0 ? a.hq / a.hkv : 0;
-    return a.cu_q_lens == nullptr && a.d == D && a.bs == BS && a.q_dtype == AICOMP_KV_BF16 &&
+    const bool shape = (a.d == D && group <= 16 && a.partition_size % TILE == 0) ||
+                       (a.d == 64 && group <= 8 && a.partition_size % (2 * TILE) == 0);
+    return a.cu_q_lens == nullptr && shape && a.bs == BS && a.q_dtype == AICOMP_KV_BF16 &&
            (a.kv_dtype == AICOMP_KV_BF16 || a.kv_dtype == AICOMP_KV_FP8_E4M3) && group >= 1 &&
-           group <= 16 && a.scale > 0.f && a.partition_size % TILE == 0 && a.rows <= 65535 &&
+           a.scale > 0.f && a.rows <= 65535 &&
            a.num_parts <= 65535 && ((uintptr_t)a.query % 16 == 0) && ((uintptr_t)a.k_pool % 16 == 0) &&
            ((uintptr_t)a.v_pool % 16 == 0);
 }
 
 bool decode_streamk_supported(const DecodeArgs& a) {
-    return decode_mfma_supported(a) && a.rows <= SK_MAX_SEQS;
+    return decode_mfma_supported(a) && a.d == D && a.rows <= SK_MAX_SEQS;
 }
 
 size_t decode_streamk_workspace_bytes(int64_t rows, int hq, int hkv, int d) {
@@ -835,10 +910,14 @@ int launch_decode_mfma(const DecodeArgs& a) {
     p.partition_size = a.partition_size; p.num_parts = a.num_parts;
     p.ws_counters = a.ws.counters; p.ws_acc = a.ws.acc; p.ws_ml = a.ws.ml;
     dim3 grid((unsigned)a.hkv, (unsigned)a.num_parts, (unsigned)a.rows);
-    if (a.kv_dtype == AICOMP_KV_FP8_E4M3)
-        hipLaunchKernelGGL(paged_decode_mfma_kernel<true>, grid, dim3(256), 0, a.stream, p);
-    else
-        hipLaunchKernelGGL(paged_decode_mfma_kernel<false>, grid, dim3(256), 0, a.stream, p);
+    const bool fp8 = a.kv_dtype == AICOMP_KV_FP8_E4M3;
+    if (a.d == 64) {
+        if (fp8) hipLaunchKernelGGL((paged_decode_mfma_kernel<true, true>), grid, dim3(256), 0, a.stream, p);
+        else hipLaunchKernelGGL((paged_decode_mfma_kernel<false, true>), grid, dim3(256), 0, a.stream, p);
+    } else {
+        if (fp8) hipLaunchKernelGGL((paged_decode_mfma_kernel<true, false>), grid, dim3(256), 0, a.stream, p);
+        else hipLaunchKernelGGL((paged_decode_mfma_kernel<false, false>), grid, dim3(256), 0, a.stream, p);
+    }
     AICOMP_HIP_LAUNCH_CHECK();
     if (a.num_parts > 1) return launch_split_reduce(a);
     return AICOMP_KV_OK;

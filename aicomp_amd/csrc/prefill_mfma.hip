@@ -102,13 +102,21 @@ template <> struct Stage<true> { uint2 k[KT / 16], v[KT / 16]; };
 // R = 16-row column groups per wave (1 or 2).  With R = 2 every K and V operand read from LDS
 // (and every V permute) feeds two MFMAs, and the two groups' softmax chains are independent, so
 // LDS traffic and permute work per flop halve and the scheduler has two chains to interleave.
-template <bool FP8, int R>
+// PAIR (head_dim 64): an LDS row is a PAIR of consecutive tokens (token 2r in elements 0..63,
+// token 2r+1 in 64..127, contiguous in the pool), a tile is 64 tokens, and every query row takes
+// two B-operand columns, one per token parity, carrying the query in the matching half of the
+// row and zeros in the other.  The two columns run independent online softmaxes and are merged
+// at the end.  Same instruction stream per byte as head_dim 128, half of it on zeros.
+template <bool FP8, int R, bool PAIR>
 __global__ void __launch_bounds__(256, R == 1 ? 3 : 2)
 paged_prefill_mfma_kernel(PrefillParams p) {
     // Grid: x = head group (fastest: the workgroups of one KV head land on one XCD and share its
     // L2 copy of that head's K/V), y = query tile, longest first (the last tile of a chunk sees
     // the most keys, so it is started first), z = sequence.
-    constexpr int WROWS = 16 * R;              // rows per wave
+    constexpr int DQ = PAIR ? 64 : D;          // head_dim of the tensors
+    constexpr int TT = PAIR ? 2 * KT : KT;     // tokens per LDS tile
+    constexpr int CR = PAIR ? 8 : 16;          // query rows per 16-column group
+    constexpr int WROWS = CR * R;              // rows per wave
     const int seq = blockIdx.z;
     const int hgroup = blockIdx.x;
     const int qtile = gridDim.y - 1 - blockIdx.y;
@@ -121,17 +129,17 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     const int n = p.cu_q_lens[seq + 1] - q_begin;
     const int ctx = min(p.context_lens[seq], p.max_blocks * BS);
     const int prior = ctx - n;
-    const int pos_per_wg = ROWS * R / p.gpack;
+    const int pos_per_wg = 4 * WROWS / p.gpack;
     const int q0 = qtile * pos_per_wg;
     if (q0 >= n || n <= 0 || prior < 0) return;
 
-    // rows of this lane's columns: row = WROWS*w + 16c + r16 -> (position, head)
+    // rows of this lane's columns: row = WROWS*w + CR*c + (column, or column / 2) -> (position, head)
     const int kvh = (hgroup * p.gpack) / p.group;          // workgroup-uniform
     int qpos[R], head[R], qabs[R];
     bool row_valid[R];
 #pragma unroll
     for (int c = 0; c < R; ++c) {
-        const int row = WROWS * w + 16 * c + r16;
+        const int row = WROWS * w + CR * c + (PAIR ? (r16 >> 1) : r16);
         qpos[c] = q0 + row / p.gpack;
         head[c] = hgroup * p.gpack + row % p.gpack;
         row_valid[c] = qpos[c] < n;
@@ -141,7 +149,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     const int wave_kv_end = min(ctx, prior + q0 + (WROWS * w + WROWS - 1) / p.gpack + 1);
     const int wave_kv_min = prior + q0 + (WROWS * w) / p.gpack;    // smallest qabs in the wave (if valid)
     const int kv_end = min(ctx, prior + q0 + pos_per_wg);
-    const int ntiles = (kv_end + KT - 1) / KT;
+    const int ntiles = (kv_end + TT - 1) / TT;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [2][K tile | V tile]
 
@@ -149,10 +157,14 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     bf16x8_t qf[R][4];
 #pragma unroll
     for (int c = 0; c < R; ++c) {
-        const uint4* qp = (const uint4*)((const bf16_t*)p.query +
-                                         ((int64_t)(q_begin + min(qpos[c], n - 1)) * p.hq + head[c]) * D + 8 * g4);
+        const bf16_t* qrow = (const bf16_t*)p.query + ((int64_t)(q_begin + min(qpos[c], n - 1)) * p.hq + head[c]) * DQ;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) qf[c][s] = __builtin_bit_cast(bf16x8_t, qp[s * 4]);
+        for (int s = 0; s < 4; ++s) {
+            const int e0 = 32 * s + 8 * g4;                     // first element of this k-slot in the LDS row
+            uint4 v = *(const uint4*)(qrow + (PAIR ? (e0 & 63) : e0));
+            if (PAIR && ((e0 >= 64) != ((r16 & 1) != 0))) v = make_uint4(0, 0, 0, 0);
+            qf[c][s] = __builtin_bit_cast(bf16x8_t, v);
+        }
     }
     // log2(e) * scale * k_scale.  The softmax below tracks the max of the raw scores, which needs
     // a positive multiplier: a negative one (a negative k_scale) moves its sign into Q.
@@ -182,15 +194,17 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
     const_i32_ptr table = (const_i32_ptr)(p.block_table + (int64_t)seq * p.block_table_stride);
 
-    // global -> registers: load i of the tile is block (KT/16)*t + i (16 tokens x 16 chunks = 256 lanes)
+    // global -> registers: load i of the tile is block (KT/16)*t + i (16 tokens x 16 chunks = 256 lanes);
+    // PAIR: a load covers two 2 KB blocks, waves 0-1 the first, waves 2-3 the second
     Stage<FP8> st;
     auto fetch = [&](int t) {
 #pragma unroll
         for (int i = 0; i < KT / 16; ++i) {
-            const int bi = (KT / 16) * t + i;
+            const int bi = PAIR ? (TT / 16) * t + 2 * i + (w >> 1) : (KT / 16) * t + i;
             int b = bi < p.max_blocks ? table[bi] : 0;
             const int64_t blk = b < 0 ? 0 : (b >= p.num_blocks ? p.num_blocks - 1 : (int64_t)b);
-            const int64_t off = (blk * p.hkv + kvh) * (BS * D / 8) + tid;
+            const int64_t off = PAIR ? (blk * p.hkv + kvh) * (BS * 64 / 8) + (tid & 127)
+                                     : (blk * p.hkv + kvh) * (BS * D / 8) + tid;
             if constexpr (FP8) {
                 st.k[i] = ((const uint2*)p.k_pool)[off];
                 st.v[i] = ((const uint2*)p.v_pool)[off];
@@ -207,12 +221,18 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         unsigned char* vb = kb + TILE_BYTES;
 #pragma unroll
         for (int i = 0; i < KT / 16; ++i) {
-            const int tok_local = 16 * i + (tid >> 4);
+            const int tok_local = 16 * i + (tid >> 4);           // LDS row
             const int off = tok_local * KROW + (tid & 15) * 16;
             uint4 kk, vv;
             if constexpr (FP8) { kk = fp8x8_to_bf16x8(st.k[i]); vv = fp8x8_to_bf16x8(st.v[i]); }
             else { kk = st.k[i]; vv = st.v[i]; }
-            if (t * KT + tok_local >= ctx) vv = make_uint4(0, 0, 0, 0);
+            if constexpr (PAIR) {
+                // chunks 8..15 of a row are the pair's second token; a token beyond the context is
+                // zeroed in K too (the other token's dot products run over the whole row)
+                if (t * TT + 2 * tok_local + ((tid & 15) >> 3) >= ctx) { kk = make_uint4(0, 0, 0, 0); vv = kk; }
+            } else {
+                if (t * KT + tok_local >= ctx) vv = make_uint4(0, 0, 0, 0);
+            }
             *(uint4*)(kb + off) = kk;
             *(uint4*)(vb + off) = vv;
         }
@@ -230,7 +250,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
 
         const unsigned char* kb = lds + buf * 2 * TILE_BYTES;
         const unsigned char* vb = kb + TILE_BYTES;
-        const int sub_start = t * KT;
+        const int sub_start = t * TT;
         if (sub_start >= wave_kv_end) continue;                        // wave-uniform: above the diagonal
 
         // ---- S^T = K Q^T: each K operand read feeds the R column groups
@@ -252,7 +272,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         // row's new maximum exceeds it by more than 2^8 after scaling: until then P is at most
         // 256, exact enough in bf16 and f32, and the accumulators need no rescale.  Only tiles that
         // cross the diagonal pay for the mask.
-        const bool need_mask = sub_start + KT - 1 > wave_kv_min;       // wave-uniform
+        const bool need_mask = sub_start + TT - 1 > wave_kv_min;       // wave-uniform
         bf16x8_t pf[R];
         float alpha[R];
         auto softmax = [&](auto mask_tag) {
@@ -265,7 +285,8 @@ paged_prefill_mfma_kernel(PrefillParams p) {
                 for (int i = 0; i < 4; ++i) { sc[i] = s0[c][i]; sc[4 + i] = s1[c][i]; }
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
-                    dead[k] = MASK && sub_start + 16 * (k >> 2) + 4 * (k & 3) + g4 > qabs[c];
+                    const int r = 16 * (k >> 2) + 4 * (k & 3) + g4;              // LDS row of this score
+                    dead[k] = MASK && sub_start + (PAIR ? 2 * r + (r16 & 1) : r) > qabs[c];
                     if (MASK && dead[k]) sc[k] = NEG_BIG;
                 }
                 float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
@@ -320,13 +341,40 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         }
     }
 
-    // lane (row r16 of column group c, g4) holds O^T[dim 32*g4 + 8*i + j][row] in O[c][j][i]
+    // lane (column r16 of column group c, g4) holds O^T[element 32*g4 + 8*i + j][column] in O[c][j][i]
 #pragma unroll
     for (int c = 0; c < R; ++c) {
         float l = lsum[c];
         l += __shfl_xor(l, 16);
         l += __shfl_xor(l, 32);
-        if (row_valid[c]) {
+        if constexpr (PAIR) {
+            // merge the row's two parity columns.  Column 2r (even tokens) has its output in
+            // elements 0..63, i.e. lanes g4 = 0, 1; column 2r+1 in elements 64..127, lanes g4 = 2, 3
+            // of the neighbouring column: lane ^ 33.
+            const float mp = __shfl_xor(m[c], 1), lp = __shfl_xor(l, 1);
+            const float mm = fmaxf(m[c], mp);
+            const float f = __builtin_amdgcn_exp2f((m[c] - mm) * cmul);
+            const float fp = __builtin_amdgcn_exp2f((mp - mm) * cmul);
+            const float lt = l * f + lp * fp;
+            const float inv = (lt > 0.f ? 1.f / lt : 0.f) * (FP8 ? p.v_scale[kvh] : 1.f);
+            const bool writer = row_valid[c] && (r16 & 1) == 0 && g4 < 2;
+            bf16_t* o = (bf16_t*)p.out + ((int64_t)(q_begin + min(qpos[c], n - 1)) * p.hq + head[c]) * DQ + 32 * g4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float v[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float mine = O[c][j][i] * f;
+                    v[j] = (mine + __shfl_xor(mine, 33)) * inv;
+                }
+                if (writer) {
+                    uint4 pk;
+                    pk.x = pack_bf16(v[0], v[1]); pk.y = pack_bf16(v[2], v[3]);
+                    pk.z = pack_bf16(v[4], v[5]); pk.w = pack_bf16(v[6], v[7]);
+                    *(uint4*)(o + 8 * i) = pk;
+                }
+            }
+        } else if (row_valid[c]) {
             const float inv = (l > 0.f ? 1.f / l : 0.f) * (FP8 ? p.v_scale[kvh] : 1.f);
             bf16_t* o = (bf16_t*)p.out + ((int64_t)(q_begin + qpos[c]) * p.hq + head[c]) * D + 32 * g4;
 #pragma unroll
@@ -342,22 +390,22 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     }
 }
 
-template <bool FP8, int R>
+template <bool FP8, int R, bool PAIR>
 static void launch_prefill_variant(const PrefillParams& p, dim3 grid, size_t lds_bytes, hipStream_t stream) {
     static bool once = false;
     if (!once) {
-        hipFuncSetAttribute((const void*)paged_prefill_mfma_kernel<FP8, R>,
+        hipFuncSetAttribute((const void*)paged_prefill_mfma_kernel<FP8, R, PAIR>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         once = true;
     }
-    hipLaunchKernelGGL((paged_prefill_mfma_kernel<FP8, R>), grid, dim3(256), lds_bytes, stream, p);
+    hipLaunchKernelGGL((paged_prefill_mfma_kernel<FP8, R, PAIR>), grid, dim3(256), lds_bytes, stream, p);
 }
 
 }  // namespace
 
 bool prefill_mfma_supported(const DecodeArgs& a, int max_q_len) {
     const int group = a.hkv > 0 ? a.hq / a.hkv : 0;
-    return a.cu_q_lens != nullptr && max_q_len > 0 && a.d == D && a.bs == BS &&
+    return a.cu_q_lens != nullptr && max_q_len > 0 && (a.d == D || a.d == 64) && a.bs == BS &&
            a.q_dtype == AICOMP_KV_BF16 &&
            (a.kv_dtype == AICOMP_KV_BF16 || a.kv_dtype == AICOMP_KV_FP8_E4M3) && group >= 1 &&
            a.scale > 0.f && a.num_seqs <= 65535 && ((uintptr_t)a.query % 16 == 0) &&
@@ -376,17 +424,26 @@ int launch_prefill_mfma(const DecodeArgs& a, int max_q_len) {
     p.qk_mul = a.scale * LOG2E;
     p.k_scale = a.k_scale; p.v_scale = a.v_scale;
     // two column groups per wave (128 rows per workgroup) once a chunk has that many rows
-    const int R = (int64_t)max_q_len * p.gpack >= 2 * ROWS ? 2 : 1;
-    const int pos_per_wg = ROWS * R / p.gpack;
+    const bool pair = a.d == 64;                       // head_dim 64: rows of token pairs, 32 query rows per workgroup
+    const int rows1 = pair ? ROWS / 2 : ROWS;
+    const int R = (int64_t)max_q_len * p.gpack >= 2 * rows1 ? 2 : 1;
+    const int pos_per_wg = rows1 * R / p.gpack;
     const int qtiles = (max_q_len + pos_per_wg - 1) / pos_per_wg;
     AICOMP_REQUIRE(qtiles <= 65535, AICOMP_KV_EINVAL, "paged_prefill_attn: grid too large");
     dim3 grid((unsigned)(a.hq / p.gpack), (unsigned)qtiles, (unsigned)a.num_seqs);
     const size_t lds_bytes = 4 * TILE_BYTES;   // double-buffered K and V tiles
     const bool fp8 = a.kv_dtype == AICOMP_KV_FP8_E4M3;
-    if (fp8 && R == 2) launch_prefill_variant<true, 2>(p, grid, lds_bytes, a.stream);
-    else if (fp8) launch_prefill_variant<true, 1>(p, grid, lds_bytes, a.stream);
-    else if (R == 2) launch_prefill_variant<false, 2>(p, grid, lds_bytes, a.stream);
-    else launch_prefill_variant<false, 1>(p, grid, lds_bytes, a.stream);
+    if (pair) {
+        if (fp8 && R == 2) launch_prefill_variant<true, 2, true>(p, grid, lds_bytes, a.stream);
+        else if (fp8) launch_prefill_variant<true, 1, true>(p, grid, lds_bytes, a.stream);
+        else if (R == 2) launch_prefill_variant<false, 2, true>(p, grid, lds_bytes, a.stream);
+        else launch_prefill_variant<false, 1, true>(p, grid, lds_bytes, a.stream);
+    } else {
+        if (fp8 && R == 2) launch_prefill_variant<true, 2, false>(p, grid, lds_bytes, a.stream);
+        else if (fp8) launch_prefill_variant<true, 1, false>(p, grid, lds_bytes, a.stream);
+        else if (R == 2) launch_prefill_variant<false, 2, false>(p, grid, lds_bytes, a.stream);
+        else launch_prefill_variant<false, 1, false>(p, grid, lds_bytes, a.stream);
+    }
     AICOMP_HIP_LAUNCH_CHECK();
     return AICOMP_KV_OK;
 }

@@ -298,3 +298,59 @@ def test_decode_all_sequences_empty(device):
     for ps in (0, 64):
         out = run_decode(w, ps, ctx=ctx)
         assert float(out.float().abs().sum()) == 0.0
+
+
+# ------------------------------------------------------------------ head_dim 64 on the matrix-core kernel
+@pytest.mark.parametrize("hq,hkv,kv", [(32, 8, torch.bfloat16), (8, 8, torch.bfloat16), (16, 2, torch.bfloat16),
+                                       (6, 2, torch.bfloat16), (32, 8, torch.float8_e4m3fn)])
+def test_decode_head_dim_64(device, hq, hkv, kv):
+    """Llama-3.2-1B-like heads (D 64): rows of token pairs on the MFMA kernel, every partitioning."""
+    sh = workloads.Shape("t", 6, hq, hkv, 64, kv_dtype=kv, kv_std=0.5, ctx_lo=1, ctx_hi=900)
+    w = workloads.make_workload("t", device=device, seed=11, shape=sh)
+    want = oracle_decode(w)
+    for ps in (0, 64, 256, 4096):
+        got = to_f64(run_decode(w, ps))
+        assert_close_attn(got, want, BF16_ATOL, BF16_RTOL, f"{hq}/{hkv} D64 {kv} ps{ps}")
+
+
+def test_decode_head_dim_64_edge_lengths_and_poison(device):
+    """Odd and even lengths around pair, block and tile boundaries; non-finite data beyond the context
+    (the second token of a half-valid pair included)."""
+    bs, hkv, d = 16, 2, 64
+    sh = workloads.Shape("t", 12, 8, hkv, d, ctx_lo=200, ctx_hi=200)
+    w = workloads.make_workload("t", device=device, seed=12, shape=sh)
+    ctx = torch.tensor([0, 1, 2, 3, 15, 16, 17, 63, 64, 65, 127, 201], dtype=torch.int32, device=device)
+    used = torch.zeros(w.k_pool.shape[0] * bs, dtype=torch.bool, device=device)
+    for b, L in enumerate(ctx.tolist()):
+        t = torch.arange(L, device=device)
+        used[w.block_table[b, t // bs].long() * bs + t % bs] = True
+    kf = w.k_pool.permute(0, 2, 1, 3).reshape(-1, hkv, d).clone()
+    vf = w.v_pool.permute(0, 2, 1, 3).reshape(-1, hkv, d).clone()
+    kf[~used] = float("nan")
+    vf[~used] = float("inf")
+    w.k_pool = kf.reshape(-1, bs, hkv, d).permute(0, 2, 1, 3).contiguous()
+    w.v_pool = vf.reshape(-1, bs, hkv, d).permute(0, 2, 1, 3).contiguous()
+    kclean = torch.nan_to_num(w.k_pool.float(), nan=0.0).to(torch.bfloat16)
+    vclean = torch.nan_to_num(w.v_pool.float(), posinf=0.0).to(torch.bfloat16)
+    want = orc.paged_decode_attn(raw(w.query), raw(kclean), raw(vclean), w.block_table.cpu().numpy(),
+                                 ctx.cpu().numpy(), w.scale, "bf16", "bf16")
+    for ps in (0, 64, 128):
+        got = to_f64(run_decode(w, ps, ctx=ctx))
+        assert_close_attn(got, want, BF16_ATOL, BF16_RTOL, f"ps {ps}")
+        assert np.array_equal(got[0], np.zeros_like(got[0]))
+        v_row = to_f64(vclean[w.block_table[1, 0].long(), :, 0, :])       # L == 1: exactly the V row
+        assert np.array_equal(got[1], np.repeat(v_row, 4, axis=0))
+
+
+def test_decode_head_dim_64_fused_append(device):
+    sh = workloads.Shape("t", 5, 32, 8, 64, kv_std=0.5, ctx_lo=1, ctx_hi=500)
+    w = workloads.make_workload("t", device=device, seed=13, shape=sh)
+    kp, vp = w.k_pool.clone(), w.v_pool.clone()
+    ops.kv_append(w.new_key, w.new_value, kp, vp, w.slot_mapping)
+    ref = torch.empty_like(w.query)
+    ops.paged_decode_attn(ref, w.query, kp, vp, w.block_table, w.context_lens, w.scale)
+    out = torch.empty_like(w.query)
+    ops.paged_decode_attn(out, w.query, w.k_pool, w.v_pool, w.block_table, w.context_lens, w.scale,
+                          new_key=w.new_key, new_value=w.new_value)
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref) and torch.equal(w.k_pool, kp) and torch.equal(w.v_pool, vp)

@@ -146,3 +146,31 @@ def test_config4_chunked_prefill_reduced(device):
             qv = orc.decode_elements(qraw[r], "bf16")[None]
             want = orc.attend_contiguous(qv, k[: prior + i + 1], v[: prior + i + 1], w.scale)[0]
             assert_close_attn(got[r], want, BF16_ATOL, BF16_RTOL, f"chunk {sidx} row {i}")
+
+
+# ------------------------------------------------------------------ head_dim 64 on the matrix-core kernel
+@pytest.mark.parametrize("hq,hkv,kv", [(8, 2, None), (4, 4, None), (32, 8, None), (6, 2, None), (16, 1, None),
+                                       (16, 2, torch.float8_e4m3fn)])
+def test_prefill_head_dim_64(device, hq, hkv, kv):
+    """Llama-3.2-1B-like heads: ragged chunks with odd priors and lengths (both token parities on the
+    diagonal), non-finite poison beyond every context."""
+    c = build_case(device, priors=[0, 5, 37, 200, 0, 63, 1], news=[70, 1, 33, 17, 1, 130, 2], hq=hq, hkv=hkv, d=64,
+                   kv_dtype=kv, seed=21)
+    got = to_f64(run(c, max_q_len=130))
+    assert_close_attn(got, oracle(c), BF16_ATOL, BF16_RTOL, f"D64 {hq}/{hkv}")
+
+
+def test_prefill_head_dim_64_long_chunks(device):
+    # two column groups per wave (chunks of >= 64 rows), several 64-token tiles, a chunk of 512
+    c = build_case(device, priors=[0, 333], news=[512, 200], hq=8, hkv=2, d=64, seed=22)
+    got = to_f64(run(c))
+    assert_close_attn(got, oracle(c), BF16_ATOL, BF16_RTOL, "D64 long")
+    # prior 0: torch's is_causal=True on the gathered K/V
+    L = 512
+    blocks = c["table"][0, : L // 16].long()
+    k = c["k_pool"][blocks].permute(1, 0, 2, 3).reshape(2, L, 64).float().cpu()
+    v = c["v_pool"][blocks].permute(1, 0, 2, 3).reshape(2, L, 64).float().cpu()
+    q = c["q"][:L].float().cpu().permute(1, 0, 2)[None]
+    want = torch.nn.functional.scaled_dot_product_attention(
+        q, k.repeat_interleave(4, 0)[None], v.repeat_interleave(4, 0)[None], is_causal=True)
+    assert_close_attn(got[:L], want[0].permute(1, 0, 2).double().numpy(), BF16_ATOL, BF16_RTOL, "causal D64")
