@@ -107,25 +107,22 @@ template <> __device__ __forceinline__ void store_elem<float>(float* p, float v)
 template <> __device__ __forceinline__ void store_elem<bf16_t>(bf16_t* p, float v) { p->bits = f32_to_bf16(v); }
 
 // ------------------------------------------------- split-K workspace view ---
-// counters [rows][Hkv] int32      : partitions finished per (row, KV head); zero between calls
 // part_acc [rows][Hq][P][D] float : sum_j 2^(s_j - m) v_j   (not normalised)
 // part_ml  [rows][Hq][P][2] float : m (log2 domain), l = sum_j 2^(s_j - m)
+// Every slot a merge reads has been written by the same call: no initialisation needed.
 struct SplitWorkspace {
-    int* counters;
     float* acc;
     float* ml;
 };
 
-inline size_t split_counter_bytes(int64_t rows, int hkv) {
-    return ((size_t)rows * hkv * sizeof(int) + 255) / 256 * 256;
-}
 inline size_t split_workspace_bytes(int64_t rows, int hq, int hkv, int d, int parts) {
-    return split_counter_bytes(rows, hkv) + (size_t)rows * hq * parts * (size_t)(d + 2) * sizeof(float);
+    (void)hkv;
+    return (size_t)rows * hq * parts * (size_t)(d + 2) * sizeof(float);
 }
 inline SplitWorkspace split_workspace_view(void* ws, int64_t rows, int hq, int hkv, int d, int parts) {
+    (void)hkv;
     SplitWorkspace v;
-    v.counters = (int*)ws;
-    v.acc = (float*)((char*)ws + split_counter_bytes(rows, hkv));
+    v.acc = (float*)ws;
     v.ml = v.acc + (size_t)rows * hq * parts * d;
     return v;
 }

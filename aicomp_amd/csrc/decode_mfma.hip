@@ -72,7 +72,6 @@ struct MfmaParams {
     const float* k_scale;
     const float* v_scale;
     int partition_size, num_parts;
-    int* ws_counters;
     float* ws_acc;
     float* ws_ml;
 };
@@ -908,7 +907,7 @@ int launch_decode_mfma(const DecodeArgs& a) {
     p.qk_mul = a.scale * LOG2E;
     p.k_scale = a.k_scale; p.v_scale = a.v_scale;
     p.partition_size = a.partition_size; p.num_parts = a.num_parts;
-    p.ws_counters = a.ws.counters; p.ws_acc = a.ws.acc; p.ws_ml = a.ws.ml;
+    p.ws_acc = a.ws.acc; p.ws_ml = a.ws.ml;
     dim3 grid((unsigned)a.hkv, (unsigned)a.num_parts, (unsigned)a.rows);
     const bool fp8 = a.kv_dtype == AICOMP_KV_FP8_E4M3;
     if (a.d == 64) {

@@ -101,7 +101,7 @@ def _workspace(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
     key = (device.index or 0, torch.cuda.current_stream(device).cuda_stream)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = torch.zeros(nbytes, dtype=torch.uint8, device=device)   # counters start at zero
+        buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
         _workspaces[key] = buf
     return buf
 

@@ -92,13 +92,11 @@ int aicomp_kv_append(const void* key, const void* value,
  *                   (max, sum, output) triples.
  *   workspace       device scratch of at least
  *                   aicomp_paged_decode_workspace_bytes(...) bytes (may be NULL
- *                   when that returns 0), 16-byte aligned.  Its leading
- *                   batch * num_kv_heads int32 words are completion counters:
- *                   they must be ZERO before the first call that uses the
- *                   buffer and every call leaves them zero again, so one
- *                   zero-filled allocation serves any number of calls.  Two
- *                   calls that may overlap (different streams) need separate
- *                   workspaces.
+ *                   when that returns 0), 16-byte aligned.  Its contents need
+ *                   no initialisation (every partial a call merges was written
+ *                   by that call) and nothing is kept in it between calls, so
+ *                   one allocation serves any number of calls.  Two calls that
+ *                   may overlap (different streams) need separate workspaces.
  */
 int aicomp_paged_decode_attn(void* out, const void* query,
                              const void* k_pool, const void* v_pool,
