@@ -52,6 +52,9 @@ SHAPES: Dict[str, Shape] = {
     # Llama-3-8B decode: batch 64, bf16, 32/8 heads, D 128, L in [512,4096]
     "llama3_8b_decode": Shape("llama3_8b_decode", 64, 32, 8, 128, kv_std=0.5,
                               ctx_lo=512, ctx_hi=4096),
+    # Llama-3.2-1B decode (the model of the reference's examples): head_dim 64, same batch and contexts
+    "llama32_1b_decode": Shape("llama32_1b_decode", 64, 32, 8, 64, kv_std=0.5,
+                               ctx_lo=512, ctx_hi=4096),
     # long-context skewed batch: batch 16, log-normal median 4096, sigma 1.0
     "long_context_skewed": Shape("long_context_skewed", 16, 32, 8, 128, kv_std=0.5,
                                  ctx="lognormal", ctx_lo=256, ctx_hi=32768,

@@ -431,7 +431,7 @@ def main():
     if not args.no_extra:
         extra = []
         for name in ("decode_fp32_small", "long_context_skewed", "chunked_prefill_mixed",
-                     "llama3_70b_decode_fp8"):
+                     "llama3_70b_decode_fp8", "llama32_1b_decode"):
             r, ww = run_decode_config(name, max(10, args.steps // 4), max(3, args.warmup // 4), dev)
             del ww
             torch.cuda.empty_cache()
