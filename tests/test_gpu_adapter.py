@@ -102,3 +102,15 @@ def test_adapter_chunked_prefill_is_causal(device):
         step = b(q1[:, :, i:i + 1], ex(k1[:, :, i:i + 1]), ex(v1[:, :, i:i + 1]))
         assert (step[:, :, 0].float() - chunk[:, :, i].float()).abs().max() <= 4e-3
     assert a.cache_pos == b.cache_pos == 29
+
+
+def test_adapter_llama32_1b_heads_bf16(device):
+    """The model of the reference's examples (Llama-3.2-1B: 32 query / 8 KV heads of 64): prefill of an
+    odd length, decode steps across a block boundary, K/V arriving expanded by repeat_kv."""
+    B, hq, g, d = 2, 32, 4, 64
+    new = akv.CachedScaledDotProductAttention(0, max_seq_len=256, dtype=torch.bfloat16)
+    ref = cref.ContiguousCachedAttention(0, 256)
+    new.enable(); ref.enable()
+    _run_session(new, ref, B, hq, g, d, [77, 1, 1, 1, 1, 1], device, torch.bfloat16, 1e-2)
+    assert new._group == 4 and new.cache_k.shape == (2 * 16, 8, 16, 64)
+    new.disable()
