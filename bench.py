@@ -83,16 +83,22 @@ def run_decode_config(name, steps, warmup, dev):
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    # HIP events cost a few microseconds of stream time each, so only every `stride`-th step
-    # of the timed region carries them (the kernel durations are averaged over those steps)
-    stride = max(1, min(8, steps // 10))
-    evs = {i: _events(4) for i in range(0, steps, stride)}
+    # Two HIP events bracket the timed region on the launch stream: with the steps queued back to
+    # back their distance / K is the average duration of a step's launches.  A step that has
+    # several phases (append, prefill, decode) also carries events between the phases, but only on
+    # ten of the steps: an event costs a few microseconds of stream time.
+    stride = max(1, steps // 10)
+    evs = {i: _events(4) for i in range(0, steps, stride)} if npre else {}
+    r_begin, r_end = _events(2)
     t0 = time.perf_counter()
+    r_begin.record()
     for i in range(steps):
         step(evs.get(i))
+    r_end.record()
     t_enqueue = time.perf_counter() - t0
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    region = r_begin.elapsed_time(r_end) / steps * 1e-3     # seconds per step, device time line
     evs = list(evs.values())
     # the stand-alone append kernel, timed on its own: 20 launches between two events, queued
     # behind ~1 ms of filler work so that the host's launch rate does not enter the figure
@@ -133,7 +139,8 @@ def run_decode_config(name, steps, warmup, dev):
     del filler
     t_app = a0.elapsed_time(a1) / 20 * 1e-3
     t_pre = statistics.mean(e[1].elapsed_time(e[2]) for e in evs) * 1e-3 if npre else 0.0
-    t_dec = statistics.mean(e[2 if npre else 1].elapsed_time(e[3]) for e in evs) * 1e-3
+    # a pure decode step is one call (main + merge kernel): its average duration is the region's
+    t_dec = statistics.mean(e[2].elapsed_time(e[3]) for e in evs) * 1e-3 if npre else region
     res = {
         "workload": name, "ms_per_step": wall / steps * 1e3,
         "host_enqueue_ms_per_step": t_enqueue / steps * 1e3,
@@ -432,7 +439,7 @@ def main():
         extra = []
         for name in ("decode_fp32_small", "long_context_skewed", "chunked_prefill_mixed",
                      "llama3_70b_decode_fp8", "llama32_1b_decode"):
-            r, ww = run_decode_config(name, max(10, args.steps // 4), max(3, args.warmup // 4), dev)
+            r, ww = run_decode_config(name, args.steps, args.warmup, dev)
             del ww
             torch.cuda.empty_cache()
             extra.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})
