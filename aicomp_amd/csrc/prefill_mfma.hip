@@ -25,10 +25,10 @@
 //              the A operand and the wave's query rows as B columns
 //              (v_mfma_f32_16x16x32_bf16); online softmax per column on the raw
 //              scores with a lazily moved max, lane-local except the row max (two
-//              lane swaps); O^T += V^T P^T with V read from LDS as 16-byte row chunks
-//              and the j-th halves picked with v_perm_b32, the same register
-//              layout as the decode kernel, so P never leaves its lane.  With two
-//              column groups every LDS operand read and permute feeds two MFMAs.
+//              lane swaps); O^T += V^T P^T with the V^T operand read out of the row-major
+//              V tile by gfx950's transposing LDS read (ds_read_b64_tr_b16), in the token
+//              order the QK product was laid out in, so P never leaves its lane.  With two
+//              column groups every LDS operand read feeds two MFMAs.
 #include "common.h"
 
 #include <type_traits>
@@ -240,7 +240,8 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     };
 
     const int rd_k = (4 * (r16 & 3) + (r16 >> 2)) * KROW + g4 * 16;   // permuted K row, chunk g4
-    const int rd_v = g4 * KROW + r16 * 16;                            // V row 4i + g4, chunk r16
+    // transposing V read: lane k of a 16-lane group addresses token row 4*(k/4) + g4, elements 4*(k%4) ..
+    const int rd_v = (4 * (r16 >> 2) + g4) * KROW + (r16 & 3) * 8;
 
     // Two register stages: tile t+2 is requested as soon as tile t has left its stage for LDS, so a
     // tile's loads have two tile steps to land.
@@ -324,22 +325,24 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             }
         }
 
-        // ---- O^T += V^T P^T: each permuted V operand feeds the R column groups
-        uint4 vv[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) vv[i] = *(const uint4*)(vb + 4 * i * KROW + rd_v);
+        // ---- O^T += V^T P^T.  The A operand (element 16j + m for lane column m, eight tokens of
+        // k-group g4) comes straight out of the row-major V tile with gfx950's transposing LDS
+        // read: within 16 lanes, lane k points at four consecutive elements of one token (token
+        // slot k/4, elements 16j + 4*(k%4) ..) and lane m receives element m%4 of the rows given
+        // by lanes 4e + m/4, e = 0..3, i.e. element 16j + m of four tokens.  Two reads (k-slots
+        // 0..3, 4..7) make one operand, which feeds the R column groups.
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
-            const uint32_t* v0 = (const uint32_t*)&vv[0];
-            uint4 a;
-            a.x = __builtin_amdgcn_perm(v0[4 * 1 + (j >> 1)], v0[4 * 0 + (j >> 1)], sel);
-            a.y = __builtin_amdgcn_perm(v0[4 * 3 + (j >> 1)], v0[4 * 2 + (j >> 1)], sel);
-            a.z = __builtin_amdgcn_perm(v0[4 * 5 + (j >> 1)], v0[4 * 4 + (j >> 1)], sel);
-            a.w = __builtin_amdgcn_perm(v0[4 * 7 + (j >> 1)], v0[4 * 6 + (j >> 1)], sel);
+            typedef short v4i16_t __attribute__((ext_vector_type(4)));
+            typedef __attribute__((address_space(3))) v4i16_t* lds_v4i16_ptr;
+            const v4i16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(vb + rd_v + j * 32));
+            const v4i16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(vb + rd_v + 16 * KROW + j * 32));
+            typedef short v8i16_t __attribute__((ext_vector_type(8)));
+            const v8i16_t av = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            const bf16x8_t a = __builtin_bit_cast(bf16x8_t, av);
 #pragma unroll
             for (int c = 0; c < R; ++c)
-                O[c][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), pf[c], O[c][j], 0, 0, 0);
+                O[c][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[c], O[c][j], 0, 0, 0);
         }
     };
     Stage<FP8> st_a, st_b;
@@ -350,7 +353,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         if (t + 1 < ntiles) step(t + 1, st_b);
     }
 
-    // lane (column r16 of column group c, g4) holds O^T[element 32*g4 + 8*i + j][column] in O[c][j][i]
+    // lane (column r16 of column group c, g4) holds O^T[element 16*j + 4*g4 + i][column] in O[c][j][i]
 #pragma unroll
     for (int c = 0; c < R; ++c) {
         float l = lsum[c];
@@ -358,43 +361,33 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         l += __shfl_xor(l, 32);
         if constexpr (PAIR) {
             // merge the row's two parity columns.  Column 2r (even tokens) has its output in
-            // elements 0..63, i.e. lanes g4 = 0, 1; column 2r+1 in elements 64..127, lanes g4 = 2, 3
-            // of the neighbouring column: lane ^ 33.
+            // elements 0..63 (j < 4), column 2r+1 in elements 64..127 (j >= 4) of the neighbouring
+            // lane.
             const float mp = __shfl_xor(m[c], 1), lp = __shfl_xor(l, 1);
             const float mm = fmaxf(m[c], mp);
             const float f = __builtin_amdgcn_exp2f((m[c] - mm) * cmul);
             const float fp = __builtin_amdgcn_exp2f((mp - mm) * cmul);
             const float lt = l * f + lp * fp;
             const float inv = (lt > 0.f ? 1.f / lt : 0.f) * (FP8 ? p.v_scale[kvh] : 1.f);
-            const bool writer = row_valid[c] && (r16 & 1) == 0 && g4 < 2;
-            bf16_t* o = (bf16_t*)p.out + ((int64_t)(q_begin + min(qpos[c], n - 1)) * p.hq + head[c]) * DQ + 32 * g4;
+            const bool writer = row_valid[c] && (r16 & 1) == 0;
+            bf16_t* o = (bf16_t*)p.out + ((int64_t)(q_begin + min(qpos[c], n - 1)) * p.hq + head[c]) * DQ + 4 * g4;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float v[8];
+            for (int j = 0; j < 4; ++j) {
+                float v[4];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const float mine = O[c][j][i] * f;
-                    v[j] = (mine + __shfl_xor(mine, 33)) * inv;
+                for (int i = 0; i < 4; ++i) {
+                    const float other = __shfl_xor(O[c][j + 4][i] * f, 1);     // the odd column's elements 64 + ..
+                    v[i] = (O[c][j][i] * f + other) * inv;
                 }
-                if (writer) {
-                    uint4 pk;
-                    pk.x = pack_bf16(v[0], v[1]); pk.y = pack_bf16(v[2], v[3]);
-                    pk.z = pack_bf16(v[4], v[5]); pk.w = pack_bf16(v[6], v[7]);
-                    *(uint4*)(o + 8 * i) = pk;
-                }
+                if (writer) *(uint2*)(o + 16 * j) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
             }
         } else if (row_valid[c]) {
             const float inv = (l > 0.f ? 1.f / l : 0.f) * (FP8 ? p.v_scale[kvh] : 1.f);
-            bf16_t* o = (bf16_t*)p.out + ((int64_t)(q_begin + qpos[c]) * p.hq + head[c]) * D + 32 * g4;
+            bf16_t* o = (bf16_t*)p.out + ((int64_t)(q_begin + qpos[c]) * p.hq + head[c]) * D + 4 * g4;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                uint4 pk;
-                pk.x = pack_bf16(O[c][0][i] * inv, O[c][1][i] * inv);
-                pk.y = pack_bf16(O[c][2][i] * inv, O[c][3][i] * inv);
-                pk.z = pack_bf16(O[c][4][i] * inv, O[c][5][i] * inv);
-                pk.w = pack_bf16(O[c][6][i] * inv, O[c][7][i] * inv);
-                *(uint4*)(o + 8 * i) = pk;
-            }
+            for (int j = 0; j < 8; ++j)
+                *(uint2*)(o + 16 * j) = make_uint2(pack_bf16(O[c][j][0] * inv, O[c][j][1] * inv),
+                                                   pack_bf16(O[c][j][2] * inv, O[c][j][3] * inv));
         }
     }
 }
