@@ -184,11 +184,11 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     }
 
     const float lazy_thr = 8.f / cmul;          // +inf for a zero multiplier: every P is 1
-    float m[R], lsum[R];
+    float m[R], lsum[R], bias[R];                // bias = -m * cmul, kept beside m
     f32x4_t O[R][8];
 #pragma unroll
     for (int c = 0; c < R; ++c) {
-        m[c] = NEG_BIG; lsum[c] = 0.f;
+        m[c] = NEG_BIG; lsum[c] = 0.f; bias[c] = -NEG_BIG * cmul;
 #pragma unroll
         for (int j = 0; j < 8; ++j) O[c][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
@@ -220,6 +220,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     auto stash = [&](int t, int buf, const Stage<FP8>& st) {
         unsigned char* kb = lds + buf * 2 * TILE_BYTES;
         unsigned char* vb = kb + TILE_BYTES;
+        const bool tail = (t + 1) * TT > ctx;                    // workgroup-uniform: only the last tile
 #pragma unroll
         for (int i = 0; i < KT / 16; ++i) {
             const int tok_local = 16 * i + (tid >> 4);           // LDS row
@@ -227,12 +228,14 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             uint4 kk, vv;
             if constexpr (FP8) { kk = fp8x8_to_bf16x8(st.k[i]); vv = fp8x8_to_bf16x8(st.v[i]); }
             else { kk = st.k[i]; vv = st.v[i]; }
-            if constexpr (PAIR) {
-                // chunks 8..15 of a row are the pair's second token; a token beyond the context is
-                // zeroed in K too (the other token's dot products run over the whole row)
-                if (t * TT + 2 * tok_local + ((tid & 15) >> 3) >= ctx) { kk = make_uint4(0, 0, 0, 0); vv = kk; }
-            } else {
-                if (t * KT + tok_local >= ctx) vv = make_uint4(0, 0, 0, 0);
+            if (tail) {
+                if constexpr (PAIR) {
+                    // chunks 8..15 of a row are the pair's second token; a token beyond the context is
+                    // zeroed in K too (the other token's dot products run over the whole row)
+                    if (t * TT + 2 * tok_local + ((tid & 15) >> 3) >= ctx) { kk = make_uint4(0, 0, 0, 0); vv = kk; }
+                } else {
+                    if (t * KT + tok_local >= ctx) vv = make_uint4(0, 0, 0, 0);
+                }
             }
             *(uint4*)(kb + off) = kk;
             *(uint4*)(vb + off) = vv;
@@ -248,7 +251,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     auto step = [&](int t, Stage<FP8>& st) {
         const int buf = t & 1;
         stash(t, buf, st);
-        if (t + 2 < ntiles) fetch(t + 2, st);
+        fetch(min(t + 2, ntiles - 1), st);      // unconditional: a static count of loads in flight
         __syncthreads();          // tile t visible; everyone is done with the buffer tile t+1 will use
 
         const unsigned char* kb = lds + buf * 2 * TILE_BYTES;
@@ -278,6 +281,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         const bool need_mask = sub_start + TT - 1 > wave_kv_min;       // wave-uniform
         bf16x8_t pf[R];
         float alpha[R];
+        bool grew[R];                                                  // wave-uniform
         auto softmax = [&](auto mask_tag) {
             constexpr bool MASK = decltype(mask_tag)::value;
 #pragma unroll
@@ -292,24 +296,30 @@ paged_prefill_mfma_kernel(PrefillParams p) {
                     dead[k] = MASK && sub_start + (PAIR ? 2 * r + (r16 & 1) : r) > qabs[c];
                     if (MASK && dead[k]) sc[k] = NEG_BIG;
                 }
-                float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
-                                 fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-                mx = xor16_max(mx);
-                mx = xor32_max(mx);
-                alpha[c] = 1.f;
-                if (mx - m[c] > lazy_thr) {
-                    alpha[c] = __builtin_amdgcn_exp2f((m[c] - mx) * cmul);
-                    m[c] = mx;
+                const float mx_lane = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
+                                            fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+                // A row's scores sit in four lanes (l, l^16, l^32, l^48), which must share one
+                // reference max.  It can only have to move if some lane's own maximum outgrows it,
+                // so the exchange, the rescale factor and the accumulator rescale (below) all sit
+                // behind one wave-uniform test that is false on almost every tile after the first.
+                grew[c] = __any(mx_lane - m[c] > lazy_thr);
+                if (grew[c]) {
+                    float mx = xor16_max(mx_lane);
+                    mx = xor32_max(mx);
+                    const bool up = mx - m[c] > lazy_thr;
+                    alpha[c] = up ? __builtin_amdgcn_exp2f((m[c] - mx) * cmul) : 1.f;
+                    m[c] = up ? mx : m[c];
+                    bias[c] = -m[c] * cmul;
+                    lsum[c] *= alpha[c];
                 }
-                const float bias = -m[c] * cmul;
-                float pr[8], psum = 0.f;
+                float pr[8], psum;
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
-                    pr[k] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[k], cmul, bias));
+                    pr[k] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[k], cmul, bias[c]));
                     if (MASK && dead[k]) pr[k] = 0.f;
-                    psum += pr[k];
+                    psum = k ? psum + pr[k] : pr[k];
                 }
-                lsum[c] = lsum[c] * alpha[c] + psum;
+                lsum[c] += psum;
                 uint4 pw;
                 pw.x = pack_bf16(pr[0], pr[1]); pw.y = pack_bf16(pr[2], pr[3]);
                 pw.z = pack_bf16(pr[4], pr[5]); pw.w = pack_bf16(pr[6], pr[7]);
@@ -319,7 +329,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         if (need_mask) softmax(std::true_type{}); else softmax(std::false_type{});
 #pragma unroll
         for (int c = 0; c < R; ++c) {
-            if (__any(alpha[c] != 1.f)) {
+            if (grew[c]) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) O[c][j] *= alpha[c];
             }
@@ -345,12 +355,16 @@ paged_prefill_mfma_kernel(PrefillParams p) {
                 O[c][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[c], O[c][j], 0, 0, 0);
         }
     };
+    // Every step issues its loads, also past the end (clamped to the last tile, never used), and
+    // the loop always runs both stages: with a fixed number of loads in flight the wait before a
+    // stage is written to LDS covers that stage's loads only, not the younger ones of the other
+    // stage.  A step past the last tile stages it again and skips the arithmetic.
     Stage<FP8> st_a, st_b;
     fetch(0, st_a);
-    if (ntiles > 1) fetch(1, st_b);
+    fetch(min(1, ntiles - 1), st_b);
     for (int t = 0; t < ntiles; t += 2) {
         step(t, st_a);
-        if (t + 1 < ntiles) step(t + 1, st_b);
+        step(t + 1, st_b);
     }
 
     // lane (column r16 of column group c, g4) holds O^T[element 16*j + 4*g4 + i][column] in O[c][j][i]
