@@ -59,7 +59,7 @@ struct PrefillParams {
     const int32_t* context_lens;
     const int32_t* cu_q_lens;
     int hq, hkv, group, gpack, max_blocks;
-    int64_t num_blocks;
+    int num_blocks;
     float qk_mul;
     const float* k_scale;
     const float* v_scale;
@@ -202,16 +202,18 @@ paged_prefill_mfma_kernel(PrefillParams p) {
 #pragma unroll
         for (int i = 0; i < KT / 16; ++i) {
             const int bi = PAIR ? (TT / 16) * t + 2 * i + (w >> 1) : (KT / 16) * t + i;
-            int b = bi < p.max_blocks ? table[bi] : 0;
-            const int64_t blk = b < 0 ? 0 : (b >= p.num_blocks ? p.num_blocks - 1 : (int64_t)b);
-            const int64_t off = PAIR ? (blk * p.hkv + kvh) * (BS * 64 / 8) + (tid & 127)
-                                     : (blk * p.hkv + kvh) * (BS * D / 8) + tid;
+            const int b = bi < p.max_blocks ? table[bi] : 0;
+            const int blk = max(0, min(b, p.num_blocks - 1));
+            // uniform 64-bit base of this head's slice of the block + a constant 32-bit lane offset
+            constexpr int ESZ = FP8 ? 1 : 2;
+            const int64_t base = ((int64_t)blk * p.hkv + kvh) * (BS * DQ * ESZ);
+            const int lane_off = (PAIR ? (tid & 127) : tid) * (8 * ESZ);
             if constexpr (FP8) {
-                st.k[i] = ((const uint2*)p.k_pool)[off];
-                st.v[i] = ((const uint2*)p.v_pool)[off];
+                st.k[i] = *(const uint2*)((const char*)p.k_pool + base + lane_off);
+                st.v[i] = *(const uint2*)((const char*)p.v_pool + base + lane_off);
             } else {
-                st.k[i] = ((const uint4*)p.k_pool)[off];
-                st.v[i] = ((const uint4*)p.v_pool)[off];
+                st.k[i] = *(const uint4*)((const char*)p.k_pool + base + lane_off);
+                st.v[i] = *(const uint4*)((const char*)p.v_pool + base + lane_off);
             }
         }
     };
@@ -436,7 +438,8 @@ int launch_prefill_mfma(const DecodeArgs& a, int max_q_len) {
     p.block_table = a.block_table; p.block_table_stride = a.block_table_stride;
     p.context_lens = a.context_lens; p.cu_q_lens = a.cu_q_lens;
     p.hq = a.hq; p.hkv = a.hkv; p.group = a.hq / a.hkv; p.max_blocks = a.max_blocks;
-    p.num_blocks = a.num_blocks;
+    AICOMP_REQUIRE(a.num_blocks <= INT32_MAX, AICOMP_KV_EINVAL, "paged_prefill_attn: num_blocks too large");
+    p.num_blocks = (int)a.num_blocks;
     p.gpack = (16 % p.group == 0) ? p.group : 1;      // heads of one KV head packed per position
     p.qk_mul = a.scale * LOG2E;
     p.k_scale = a.k_scale; p.v_scale = a.v_scale;
