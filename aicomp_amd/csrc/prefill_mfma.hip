@@ -43,10 +43,8 @@ namespace {
 
 constexpr int D = 128;
 constexpr int BS = 16;
-constexpr int KT = 32;                 // tokens per LDS tile (two blocks)
 constexpr int ROWS = 64;               // query rows per workgroup and column group (16 per wave)
 constexpr int KROW = 272;              // LDS row stride in bytes (256 + 16 pad)
-constexpr int TILE_BYTES = KT * KROW;  // 8704
 constexpr float NEG_BIG = -1.0e30f;
 
 struct PrefillParams {
@@ -95,9 +93,9 @@ __device__ __forceinline__ float xor32_max(float x) {
     return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 
-template <bool FP8> struct Stage;
-template <> struct Stage<false> { uint4 k[KT / 16], v[KT / 16]; };
-template <> struct Stage<true> { uint2 k[KT / 16], v[KT / 16]; };
+template <bool FP8, int KT> struct Stage;
+template <int KT> struct Stage<false, KT> { uint4 k[KT / 16], v[KT / 16]; };
+template <int KT> struct Stage<true, KT> { uint2 k[KT / 16], v[KT / 16]; };
 
 // R = 16-row column groups per wave (1 or 2).  With R = 2 every K and V operand read from LDS
 // (and every V permute) feeds two MFMAs, and the two groups' softmax chains are independent, so
@@ -107,9 +105,16 @@ template <> struct Stage<true> { uint2 k[KT / 16], v[KT / 16]; };
 // two B-operand columns, one per token parity, carrying the query in the matching half of the
 // row and zeros in the other.  The two columns run independent online softmaxes and are merged
 // at the end.  Same instruction stream per byte as head_dim 128, half of it on zeros.
+// KT = rows of an LDS tile (KT/16 blocks): 32 with two register stages for R = 1, 64 with one stage
+// for R = 2, where the per-step work that does not scale with the tile (barrier, block lookups,
+// loop control, the running-max test) is paid half as often.
 template <bool FP8, int R, bool PAIR>
 __global__ void __launch_bounds__(256, R == 1 ? 3 : 2)
 paged_prefill_mfma_kernel(PrefillParams p) {
+    constexpr int KT = R == 1 ? 32 : 64;
+    constexpr int NH = KT / 16;                // 16-row groups of a tile
+    constexpr int TILE_BYTES = KT * KROW;
+    typedef Stage<FP8, KT> StageT;
     // Grid: x = head group (fastest: the workgroups of one KV head land on one XCD and share its
     // L2 copy of that head's K/V), y = sequence, z = query tile, longest first (the last tile of a
     // chunk sees the most keys, so it is started first).  Sequence before tile: workgroups that
@@ -197,12 +202,27 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     const_i32_ptr table = (const_i32_ptr)(p.block_table + (int64_t)seq * p.block_table_stride);
 
     // global -> registers: load i of the tile is block (KT/16)*t + i (16 tokens x 16 chunks = 256 lanes);
-    // PAIR: a load covers two 2 KB blocks, waves 0-1 the first, waves 2-3 the second
-    auto fetch = [&](int t, Stage<FP8>& st) {
+    // PAIR: a load covers two 2 KB blocks, waves 0-1 the first, waves 2-3 the second.  The block
+    // ids of a tile are consecutive table entries: one scalar load when all of them exist.
+    constexpr int NB = PAIR ? TT / 16 : KT / 16;               // table entries per tile
+    auto fetch = [&](int t, StageT& st) {
+        int ids[NB];
+        const int first = NB * t;
+        if (first + NB <= p.max_blocks) {
+            typedef int idvec_t __attribute__((ext_vector_type(NB), aligned(4)));
+            typedef const __attribute__((address_space(4))) idvec_t* const_idvec_ptr;
+            const idvec_t v = *(const_idvec_ptr)(table + first);
+#pragma unroll
+            for (int i = 0; i < NB; ++i) ids[i] = v[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < NB; ++i) ids[i] = first + i < p.max_blocks ? table[first + i] : 0;
+        }
 #pragma unroll
         for (int i = 0; i < KT / 16; ++i) {
-            const int bi = PAIR ? (TT / 16) * t + 2 * i + (w >> 1) : (KT / 16) * t + i;
-            const int b = bi < p.max_blocks ? table[bi] : 0;
+            int b;
+            if constexpr (PAIR) b = (w >> 1) ? ids[2 * i + 1] : ids[2 * i];
+            else b = ids[i];
             const int blk = max(0, min(b, p.num_blocks - 1));
             // uniform 64-bit base of this head's slice of the block + a constant 32-bit lane offset
             constexpr int ESZ = FP8 ? 1 : 2;
@@ -217,12 +237,14 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             }
         }
     };
-    // registers -> LDS buffer `buf`; V rows at or beyond the context are zeroed (a masked
-    // probability of 0 times a non-finite leftover would still poison the row)
-    auto stash = [&](int t, int buf, const Stage<FP8>& st) {
+    // registers -> LDS buffer `buf`.  On the tile that reaches the end of the context, V rows at
+    // or beyond it are zeroed (a masked probability of 0 times a non-finite leftover would still
+    // poison the row); PAIR zeroes K there too (the other token of the pair runs its dot products
+    // over the whole row).
+    auto stash_rows = [&](int t, int buf, const StageT& st, auto tail_tag) {
+        constexpr bool TAIL = decltype(tail_tag)::value;
         unsigned char* kb = lds + buf * 2 * TILE_BYTES;
         unsigned char* vb = kb + TILE_BYTES;
-        const bool tail = (t + 1) * TT > ctx;                    // workgroup-uniform: only the last tile
 #pragma unroll
         for (int i = 0; i < KT / 16; ++i) {
             const int tok_local = 16 * i + (tid >> 4);           // LDS row
@@ -230,30 +252,33 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             uint4 kk, vv;
             if constexpr (FP8) { kk = fp8x8_to_bf16x8(st.k[i]); vv = fp8x8_to_bf16x8(st.v[i]); }
             else { kk = st.k[i]; vv = st.v[i]; }
-            if (tail) {
-                if constexpr (PAIR) {
-                    // chunks 8..15 of a row are the pair's second token; a token beyond the context is
-                    // zeroed in K too (the other token's dot products run over the whole row)
-                    if (t * TT + 2 * tok_local + ((tid & 15) >> 3) >= ctx) { kk = make_uint4(0, 0, 0, 0); vv = kk; }
-                } else {
-                    if (t * KT + tok_local >= ctx) vv = make_uint4(0, 0, 0, 0);
-                }
+            if constexpr (TAIL && PAIR) {
+                // chunks 8..15 of a row are the pair's second token
+                if (t * TT + 2 * tok_local + ((tid & 15) >> 3) >= ctx) { kk = make_uint4(0, 0, 0, 0); vv = kk; }
+            } else if constexpr (TAIL) {
+                if (t * KT + tok_local >= ctx) vv = make_uint4(0, 0, 0, 0);
             }
             *(uint4*)(kb + off) = kk;
             *(uint4*)(vb + off) = vv;
         }
+    };
+    auto stash = [&](int t, int buf, const StageT& st) {
+        if ((t + 1) * TT > ctx) stash_rows(t, buf, st, std::true_type{});     // workgroup-uniform
+        else stash_rows(t, buf, st, std::false_type{});
     };
 
     const int rd_k = (4 * (r16 & 3) + (r16 >> 2)) * KROW + g4 * 16;   // permuted K row, chunk g4
     // transposing V read: lane k of a 16-lane group addresses token row 4*(k/4) + g4, elements 4*(k%4) ..
     const int rd_v = (4 * (r16 >> 2) + g4) * KROW + (r16 & 3) * 8;
 
-    // Two register stages: tile t+2 is requested as soon as tile t has left its stage for LDS, so a
-    // tile's loads have two tile steps to land.
-    auto step = [&](int t, Stage<FP8>& st) {
+    // The next tile of a stage is requested as soon as the stage has been written to LDS (two
+    // stages of 32 rows: tile t+2; one stage of 64 rows: tile t+1), so a tile's loads have the
+    // time of 64 rows of arithmetic to land.
+    constexpr int AHEAD = KT == 32 ? 2 : 1;
+    auto step = [&](int t, StageT& st) {
         const int buf = t & 1;
         stash(t, buf, st);
-        fetch(min(t + 2, ntiles - 1), st);      // unconditional: a static count of loads in flight
+        fetch(min(t + AHEAD, ntiles - 1), st);  // unconditional: a static count of loads in flight
         __syncthreads();          // tile t visible; everyone is done with the buffer tile t+1 will use
 
         const unsigned char* kb = lds + buf * 2 * TILE_BYTES;
@@ -262,18 +287,22 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         if (sub_start >= wave_kv_end) return;                          // wave-uniform: above the diagonal
 
         // ---- S^T = K Q^T: each K operand read feeds the R column groups
-        f32x4_t s0[R], s1[R];
+        f32x4_t sa[NH][R];
 #pragma unroll
-        for (int c = 0; c < R; ++c) { s0[c] = f32x4_t{0.f, 0.f, 0.f, 0.f}; s1[c] = f32x4_t{0.f, 0.f, 0.f, 0.f}; }
+        for (int h = 0; h < NH; ++h)
+#pragma unroll
+            for (int c = 0; c < R; ++c) sa[h][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            const bf16x8_t a0 = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kb + rd_k + s * 64));
-            const bf16x8_t a1 = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kb + 16 * KROW + rd_k + s * 64));
+            bf16x8_t a[NH];
 #pragma unroll
-            for (int c = 0; c < R; ++c) {
-                s0[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[c][s], s0[c], 0, 0, 0);
-                s1[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qf[c][s], s1[c], 0, 0, 0);
-            }
+            for (int h = 0; h < NH; ++h)
+                a[h] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kb + 16 * h * KROW + rd_k + s * 64));
+#pragma unroll
+            for (int h = 0; h < NH; ++h)
+#pragma unroll
+                for (int c = 0; c < R; ++c)
+                    sa[h][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[h], qf[c][s], sa[h][c], 0, 0, 0);
         }
         // Online softmax on the raw scores: the score multiplier is folded into the exponent's
         // fused multiply-add and the running max stays in raw units.  The max is only moved when a
@@ -281,25 +310,29 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         // 256, exact enough in bf16 and f32, and the accumulators need no rescale.  Only tiles that
         // cross the diagonal pay for the mask.
         const bool need_mask = sub_start + TT - 1 > wave_kv_min;       // wave-uniform
-        bf16x8_t pf[R];
+        bf16x8_t pf[R][NH / 2];
         float alpha[R];
         bool grew[R];                                                  // wave-uniform
         auto softmax = [&](auto mask_tag) {
             constexpr bool MASK = decltype(mask_tag)::value;
 #pragma unroll
             for (int c = 0; c < R; ++c) {
-                float sc[8];
-                bool dead[8];
+                constexpr int NS = 4 * NH;                                      // scores per lane
+                float sc[NS];
+                bool dead[NS];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) { sc[i] = s0[c][i]; sc[4 + i] = s1[c][i]; }
+                for (int k = 0; k < NS; ++k) sc[k] = sa[k >> 2][c][k & 3];
 #pragma unroll
-                for (int k = 0; k < 8; ++k) {
+                for (int k = 0; k < NS; ++k) {
                     const int r = 16 * (k >> 2) + 4 * (k & 3) + g4;              // LDS row of this score
                     dead[k] = MASK && sub_start + (PAIR ? 2 * r + (r16 & 1) : r) > qabs[c];
                     if (MASK && dead[k]) sc[k] = NEG_BIG;
                 }
-                const float mx_lane = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
-                                            fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+                float mx_lane = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
+                                      fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+                if constexpr (NS == 16)
+                    mx_lane = fmaxf(mx_lane, fmaxf(fmaxf(fmaxf(sc[8], sc[9]), fmaxf(sc[10], sc[11])),
+                                                   fmaxf(fmaxf(sc[12], sc[13]), fmaxf(sc[14], sc[15]))));
                 // A row's scores sit in four lanes (l, l^16, l^32, l^48), which must share one
                 // reference max.  It can only have to move if some lane's own maximum outgrows it,
                 // so the exchange, the rescale factor and the accumulator rescale (below) all sit
@@ -314,18 +347,21 @@ paged_prefill_mfma_kernel(PrefillParams p) {
                     bias[c] = -m[c] * cmul;
                     lsum[c] *= alpha[c];
                 }
-                float pr[8], psum;
+                float pr[NS], psum;
 #pragma unroll
-                for (int k = 0; k < 8; ++k) {
+                for (int k = 0; k < NS; ++k) {
                     pr[k] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[k], cmul, bias[c]));
                     if (MASK && dead[k]) pr[k] = 0.f;
                     psum = k ? psum + pr[k] : pr[k];
                 }
                 lsum[c] += psum;
-                uint4 pw;
-                pw.x = pack_bf16(pr[0], pr[1]); pw.y = pack_bf16(pr[2], pr[3]);
-                pw.z = pack_bf16(pr[4], pr[5]); pw.w = pack_bf16(pr[6], pr[7]);
-                pf[c] = __builtin_bit_cast(bf16x8_t, pw);
+#pragma unroll
+                for (int hp = 0; hp < NH / 2; ++hp) {
+                    uint4 pw;
+                    pw.x = pack_bf16(pr[8 * hp + 0], pr[8 * hp + 1]); pw.y = pack_bf16(pr[8 * hp + 2], pr[8 * hp + 3]);
+                    pw.z = pack_bf16(pr[8 * hp + 4], pr[8 * hp + 5]); pw.w = pack_bf16(pr[8 * hp + 6], pr[8 * hp + 7]);
+                    pf[c][hp] = __builtin_bit_cast(bf16x8_t, pw);
+                }
             }
         };
         if (need_mask) softmax(std::true_type{}); else softmax(std::false_type{});
@@ -347,26 +383,36 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         for (int j = 0; j < 8; ++j) {
             typedef short v4i16_t __attribute__((ext_vector_type(4)));
             typedef __attribute__((address_space(3))) v4i16_t* lds_v4i16_ptr;
-            const v4i16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(vb + rd_v + j * 32));
-            const v4i16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(vb + rd_v + 16 * KROW + j * 32));
             typedef short v8i16_t __attribute__((ext_vector_type(8)));
-            const v8i16_t av = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            const bf16x8_t a = __builtin_bit_cast(bf16x8_t, av);
 #pragma unroll
-            for (int c = 0; c < R; ++c)
-                O[c][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[c], O[c][j], 0, 0, 0);
+            for (int hp = 0; hp < NH / 2; ++hp) {
+                const unsigned char* vt = vb + 32 * hp * KROW + rd_v + j * 32;
+                const v4i16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)vt);
+                const v4i16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(vt + 16 * KROW));
+                const v8i16_t av = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                const bf16x8_t a = __builtin_bit_cast(bf16x8_t, av);
+#pragma unroll
+                for (int c = 0; c < R; ++c)
+                    O[c][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[c][hp], O[c][j], 0, 0, 0);
+            }
         }
     };
-    // Every step issues its loads, also past the end (clamped to the last tile, never used), and
-    // the loop always runs both stages: with a fixed number of loads in flight the wait before a
-    // stage is written to LDS covers that stage's loads only, not the younger ones of the other
-    // stage.  A step past the last tile stages it again and skips the arithmetic.
-    Stage<FP8> st_a, st_b;
-    fetch(0, st_a);
-    fetch(min(1, ntiles - 1), st_b);
-    for (int t = 0; t < ntiles; t += 2) {
-        step(t, st_a);
-        step(t + 1, st_b);
+    // Every step issues its loads, also past the end (clamped to the last tile, never used): with
+    // a fixed number of loads in flight the wait before a stage is written to LDS covers that
+    // stage's loads only, not the younger ones of the other stage.  With two stages the loop
+    // always runs both; a step past the last tile stages it again and skips the arithmetic.
+    if constexpr (KT == 32) {
+        StageT st_a, st_b;
+        fetch(0, st_a);
+        fetch(min(1, ntiles - 1), st_b);
+        for (int t = 0; t < ntiles; t += 2) {
+            step(t, st_a);
+            step(t + 1, st_b);
+        }
+    } else {
+        StageT st;
+        fetch(0, st);
+        for (int t = 0; t < ntiles; ++t) step(t, st);
     }
 
     // lane (column r16 of column group c, g4) holds O^T[element 16*j + 4*g4 + i][column] in O[c][j][i]
@@ -451,7 +497,7 @@ int launch_prefill_mfma(const DecodeArgs& a, int max_q_len) {
     const int qtiles = (max_q_len + pos_per_wg - 1) / pos_per_wg;
     AICOMP_REQUIRE(qtiles <= 65535, AICOMP_KV_EINVAL, "paged_prefill_attn: grid too large");
     dim3 grid((unsigned)(a.hq / p.gpack), (unsigned)a.num_seqs, (unsigned)qtiles);
-    const size_t lds_bytes = 4 * TILE_BYTES;   // double-buffered K and V tiles
+    const size_t lds_bytes = (size_t)4 * (R == 1 ? 32 : 64) * KROW;   // double-buffered K and V tiles
     const bool fp8 = a.kv_dtype == AICOMP_KV_FP8_E4M3;
     if (pair) {
         if (fp8 && R == 2) launch_prefill_variant<true, 2, true>(p, grid, lds_bytes, a.stream);
