@@ -113,6 +113,16 @@ def decode_partition_size(batch: int, hq: int, hkv: int, d: int, bs: int, max_bl
                                                   _DT[q_dtype], _DT[kv_dtype])
 
 
+def decode_workspace_bytes(batch: int, hq: int, hkv: int, d: int, bs: int, max_blocks: int,
+                           q_dtype: torch.dtype, kv_dtype: torch.dtype, partition_size: int = 0) -> int:
+    """Scratch bytes ``paged_decode_attn`` needs for these shapes.  A caller that must not allocate
+    inside the call (a step recorded into a HIP graph) allocates this once and passes it as
+    ``workspace``; the buffer needs no initialisation."""
+    lib = _lib.load()
+    return lib.aicomp_paged_decode_workspace_bytes(batch, hq, hkv, d, bs, max_blocks, _DT[q_dtype],
+                                                   _DT[kv_dtype], partition_size)
+
+
 def paged_decode_attn(out: torch.Tensor, query: torch.Tensor, k_pool: torch.Tensor,
                       v_pool: torch.Tensor, block_table: torch.Tensor,
                       context_lens: torch.Tensor, scale: float,

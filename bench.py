@@ -137,6 +137,30 @@ def run_decode_config(name, steps, warmup, dev):
     torch.cuda.synchronize()
     t_cold = statistics.median(a.elapsed_time(b) for a, b in cold) * 1e-3
     del filler
+    # the same decode step recorded once into a HIP graph and replayed: no host launch cost per step
+    # (the library allocates nothing and clears nothing, the scratch is passed in)
+    t_graph = None
+    if not npre:
+        try:
+            need = ops.decode_workspace_bytes(S, w.shape.num_q_heads, w.shape.num_kv_heads, w.shape.head_dim,
+                                              w.shape.block_size, btd.shape[1], qd.dtype, w.k_pool.dtype)
+            ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                ops.paged_decode_attn(outd, qd, w.k_pool, w.v_pool, btd, cld, w.scale, w.k_scale, w.v_scale,
+                                      new_key=nk_dec, new_value=nv_dec, workspace=ws)
+            for _ in range(3):
+                graph.replay()
+            g0, g1 = _events(2)
+            g0.record()
+            for _ in range(steps):
+                graph.replay()
+            g1.record()
+            torch.cuda.synchronize()
+            t_graph = g0.elapsed_time(g1) / steps * 1e-3
+            del graph
+        except Exception as e:                              # a bench figure, not a requirement
+            print(f"graph replay not measured for {name}: {e}", file=sys.stderr)
     t_app = a0.elapsed_time(a1) / 20 * 1e-3
     t_pre = statistics.mean(e[1].elapsed_time(e[2]) for e in evs) * 1e-3 if npre else 0.0
     # a pure decode step is one call (main + merge kernel): its average duration is the region's
@@ -153,6 +177,7 @@ def run_decode_config(name, steps, warmup, dev):
         "decode_frac_hbm_peak": w.decode_kv_bytes() / t_dec / 1e9 / HBM_PEAK_GBS,
         "decode_tokens_per_s": (S - npre) / t_dec,
         "decode_cold_us": t_cold * 1e6, "decode_cold_GBs": w.decode_kv_bytes() / t_cold / 1e9,
+        "decode_graph_replay_us": None if t_graph is None else t_graph * 1e6,
         "partition_size": ops.decode_partition_size(S - npre, w.shape.num_q_heads, w.shape.num_kv_heads,
                                                     w.shape.head_dim, w.shape.block_size, btd.shape[1],
                                                     qd.dtype, w.k_pool.dtype),
@@ -425,6 +450,7 @@ def main():
                      "avg_launch_us": main_res["decode_us"]},
         "append": {"us": main_res["append_us"], "GB/s": main_res["append_GBs"],
                    "bytes": main_res["append_bytes"]},
+        "decode_graph_replay_us": main_res["decode_graph_replay_us"],
         "decode_cold": {"us": main_res["decode_cold_us"], "GB/s": main_res["decode_cold_GBs"],
                         "note": "decode call timed right after 1 GiB of unrelated writes"},
         "device": device_info(),
