@@ -261,6 +261,46 @@ def sampler_bench(dev, batch=64, vocab=128256, temperature=0.8, top_k=50, top_p=
     return res
 
 
+def prefill_shapes_bench(dev, reps=5):
+    """The chunked-prefill kernel on shapes with many more workgroups than the named mixed step
+    (512 workgroups there, two per CU, bounded by the longest of them): fresh long prompts and a
+    batch of chunks with prior context.  Synthetic bf16 K/V, 32/8 heads, D 128."""
+    import math
+    import torch
+    from aicomp_amd import ops
+    hq, hkv, d = 32, 8, 128
+    out = []
+    for nseq, n, prior in ((1, 8192, 0), (4, 4096, 0), (16, 512, 2048)):
+        ctx = prior + n
+        nblk = math.ceil(ctx / 16)
+        nb = nseq * nblk + 1
+        g = torch.Generator().manual_seed(0)
+        table = torch.randperm(nb - 1, generator=g)[: nseq * nblk].reshape(nseq, nblk).to(torch.int32).to(dev)
+        k = (torch.randn(nb, hkv, 16, d, device=dev) * 0.5).to(torch.bfloat16)
+        v = (torch.randn(nb, hkv, 16, d, device=dev) * 0.5).to(torch.bfloat16)
+        q = torch.randn(nseq * n, hq, d, device=dev).to(torch.bfloat16)
+        o = torch.empty_like(q)
+        cl = torch.full((nseq,), ctx, dtype=torch.int32, device=dev)
+        cu = (torch.arange(nseq + 1, dtype=torch.int32) * n).to(dev)
+        call = lambda: ops.paged_prefill_attn(o, q, k, v, table, cl, cu, 1 / math.sqrt(d), max_q_len=n)
+        for _ in range(2):
+            call()
+        e0, e1 = _events(2)
+        e0.record()
+        for _ in range(reps):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) / reps * 1e-3
+        flops = nseq * 4 * hq * d * (n * prior + n * (n + 1) / 2)
+        out.append({"chunks": nseq, "new_tokens": n, "prior": prior, "us": round(t * 1e6, 1),
+                    "TFLOPs": round(flops / t / 1e12, 1),
+                    "frac_mfma_peak": round(flops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
+        del k, v, q, o
+        torch.cuda.empty_cache()
+    return out
+
+
 def device_info():
     import torch
     p = torch.cuda.get_device_properties(0)
@@ -456,6 +496,7 @@ def main():
         "device": device_info(),
         "step_planner": planner_bench(dev),
         "sampler": sampler_bench(dev),
+        "prefill_other_shapes": prefill_shapes_bench(dev),
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(w)
