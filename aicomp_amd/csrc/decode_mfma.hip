@@ -41,6 +41,8 @@
 //              workspace; a second, small kernel merges them.
 #include "common.h"
 
+#include <atomic>
+
 namespace aicomp {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -856,7 +858,10 @@ size_t decode_streamk_workspace_bytes(int64_t rows, int hq, int hkv, int d) {
 }
 
 int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
-    static int num_cus = 0;
+    // CU count of the first device used (every GPU of a node is the same part); an atomic so that
+    // callers on several threads may race here harmlessly
+    static std::atomic<int> cached_cus{0};
+    int num_cus = cached_cus.load(std::memory_order_relaxed);
     if (num_cus == 0) {
         int dev = 0, n = 0;
         if (hipGetDevice(&dev) != hipSuccess ||
@@ -865,6 +870,7 @@ int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
             return AICOMP_KV_EHIP;
         }
         num_cus = n;
+        cached_cus.store(n, std::memory_order_relaxed);
     }
     // one workgroup per CU measured fastest (4 waves of 16 KB in flight each already cover the
     // HBM latency; a second workgroup per CU only adds partials and start-up work)

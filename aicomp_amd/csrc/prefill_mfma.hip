@@ -31,6 +31,7 @@
 //              column groups every LDS operand read feeds two MFMAs.
 #include "common.h"
 
+#include <atomic>
 #include <type_traits>
 
 namespace aicomp {
@@ -455,15 +456,22 @@ paged_prefill_mfma_kernel(PrefillParams p) {
 }
 
 template <bool FP8, int R, bool PAIR>
-static void launch_prefill_variant(const PrefillParams& p, dim3 grid, size_t lds_bytes, hipStream_t stream) {
-    static bool once = false;
-    if (!once) {
-        // 34 KB of dynamic LDS is within the default limit; raising it is only a precaution
-        (void)hipFuncSetAttribute((const void*)paged_prefill_mfma_kernel<FP8, R, PAIR>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        once = true;
+static hipError_t launch_prefill_variant(const PrefillParams& p, dim3 grid, size_t lds_bytes, hipStream_t stream) {
+    // Two column groups stage 64-row tiles: 70 KB of dynamic LDS, above the 64 KB a kernel may use
+    // without asking.  The limit is a per-device function attribute: set once per device.
+    static std::atomic<unsigned long long> done{0};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const bool known = dev < 64 && ((done.load(std::memory_order_acquire) >> dev) & 1ull);
+    if (!known) {
+        e = hipFuncSetAttribute((const void*)paged_prefill_mfma_kernel<FP8, R, PAIR>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return e;
+        if (dev < 64) done.fetch_or(1ull << dev, std::memory_order_release);
     }
     hipLaunchKernelGGL((paged_prefill_mfma_kernel<FP8, R, PAIR>), grid, dim3(256), lds_bytes, stream, p);
+    return hipSuccess;
 }
 
 }  // namespace
@@ -499,17 +507,19 @@ int launch_prefill_mfma(const DecodeArgs& a, int max_q_len) {
     dim3 grid((unsigned)(a.hq / p.gpack), (unsigned)a.num_seqs, (unsigned)qtiles);
     const size_t lds_bytes = (size_t)4 * (R == 1 ? 32 : 64) * KROW;   // double-buffered K and V tiles
     const bool fp8 = a.kv_dtype == AICOMP_KV_FP8_E4M3;
+    hipError_t e;
     if (pair) {
-        if (fp8 && R == 2) launch_prefill_variant<true, 2, true>(p, grid, lds_bytes, a.stream);
-        else if (fp8) launch_prefill_variant<true, 1, true>(p, grid, lds_bytes, a.stream);
-        else if (R == 2) launch_prefill_variant<false, 2, true>(p, grid, lds_bytes, a.stream);
-        else launch_prefill_variant<false, 1, true>(p, grid, lds_bytes, a.stream);
+        if (fp8 && R == 2) e = launch_prefill_variant<true, 2, true>(p, grid, lds_bytes, a.stream);
+        else if (fp8) e = launch_prefill_variant<true, 1, true>(p, grid, lds_bytes, a.stream);
+        else if (R == 2) e = launch_prefill_variant<false, 2, true>(p, grid, lds_bytes, a.stream);
+        else e = launch_prefill_variant<false, 1, true>(p, grid, lds_bytes, a.stream);
     } else {
-        if (fp8 && R == 2) launch_prefill_variant<true, 2, false>(p, grid, lds_bytes, a.stream);
-        else if (fp8) launch_prefill_variant<true, 1, false>(p, grid, lds_bytes, a.stream);
-        else if (R == 2) launch_prefill_variant<false, 2, false>(p, grid, lds_bytes, a.stream);
-        else launch_prefill_variant<false, 1, false>(p, grid, lds_bytes, a.stream);
+        if (fp8 && R == 2) e = launch_prefill_variant<true, 2, false>(p, grid, lds_bytes, a.stream);
+        else if (fp8) e = launch_prefill_variant<true, 1, false>(p, grid, lds_bytes, a.stream);
+        else if (R == 2) e = launch_prefill_variant<false, 2, false>(p, grid, lds_bytes, a.stream);
+        else e = launch_prefill_variant<false, 1, false>(p, grid, lds_bytes, a.stream);
     }
+    AICOMP_REQUIRE(e == hipSuccess, AICOMP_KV_EHIP, "paged_prefill_attn: %s", hipGetErrorString(e));
     AICOMP_HIP_LAUNCH_CHECK();
     return AICOMP_KV_OK;
 }
