@@ -58,6 +58,19 @@ def _detect_group(key: torch.Tensor) -> int:
     return 1
 
 
+_CTX_ROWS: Dict[tuple, torch.Tensor] = {}
+
+
+def _ctx_rows(rows: int, batch: int, device: torch.device) -> torch.Tensor:
+    """``[rows, batch]`` int32 with row L filled with L; one tensor per geometry, shared by the layers."""
+    key = (device.type, device.index, rows, batch)
+    t = _CTX_ROWS.get(key)
+    if t is None:
+        t = torch.arange(rows, dtype=torch.int32, device=device)[:, None].expand(-1, batch).contiguous()
+        _CTX_ROWS[key] = t
+    return t
+
+
 class _PagedLayer:
     """K and V block pools of one layer plus the static tables of a fixed batch."""
 
@@ -76,6 +89,10 @@ class _PagedLayer:
         base = torch.arange(batch, dtype=torch.int64, device=device) * (self.blocks_per_seq * block_size)
         self.slot_table = base[:, None] + t[None, :]                       # [B, padded max_seq]
         self.context_lens = torch.zeros(batch, dtype=torch.int32, device=device)
+        # row L of this table is the context-length vector of a step that sees L tokens: all
+        # sequences share one position, so a decode step takes a view instead of launching a fill
+        self.ctx_rows = _ctx_rows(self.blocks_per_seq * block_size + 1, batch, torch.device(device))
+        self._decode: Dict[tuple, ops.PreparedDecode] = {}
         self.cu_q_lens = torch.zeros(batch + 1, dtype=torch.int32, device=device)
         self._cu_n = -1
 
@@ -102,11 +119,14 @@ class _PagedLayer:
         B, Hq, _, D = query.shape
         if key.shape[1] == self.kv_heads * group and group > 1:
             key, value = key[:, ::group], value[:, ::group]
-        self.context_lens.fill_(pos + 1)
+        call = self._decode.get((Hq, query.dtype, scale))
+        if call is None:
+            call = ops.PreparedDecode(self.k_pool, self.v_pool, self.block_table, self.context_lens, Hq,
+                                      query.dtype, scale)
+            self._decode[(Hq, query.dtype, scale)] = call
         q = query[:, :, 0, :].contiguous()
         out = torch.empty_like(q)
-        ops.paged_decode_attn(out, q, self.k_pool, self.v_pool, self.block_table, self.context_lens,
-                              scale, new_key=key[:, :, 0, :], new_value=value[:, :, 0, :])
+        call(out, q, key[:, :, 0, :], value[:, :, 0, :], context_lens=self.ctx_rows[pos + 1])
         return out.view(B, Hq, 1, D)
 
     def attend(self, query: torch.Tensor, pos: int, scale: float) -> torch.Tensor:
@@ -122,7 +142,8 @@ class _PagedLayer:
         if self._cu_n != n:
             self.cu_q_lens.copy_(torch.arange(B + 1, dtype=torch.int32, device=query.device) * n)
             self._cu_n = n
-        q = query.permute(0, 2, 1, 3).reshape(B * n, Hq, D)
+        # token-major rows; for batch 1 the reshape is a strided view, hence the explicit copy
+        q = query.permute(0, 2, 1, 3).reshape(B * n, Hq, D).contiguous()
         out = torch.empty_like(q)
         ops.paged_prefill_attn(out, q, self.k_pool, self.v_pool, self.block_table,
                                self.context_lens, self.cu_q_lens, scale, max_q_len=n)

@@ -95,10 +95,10 @@ def kv_append(key: torch.Tensor, value: torch.Tensor, k_pool: torch.Tensor, v_po
 _workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
 
 
-def _workspace(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
+def _workspace(device: torch.device, nbytes: int, stream: Optional[int] = None) -> Optional[torch.Tensor]:
     if nbytes == 0:
         return None
-    key = (device.index or 0, torch.cuda.current_stream(device).cuda_stream)
+    key = (device.index or 0, torch.cuda.current_stream(device).cuda_stream if stream is None else stream)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
@@ -186,6 +186,77 @@ def paged_decode_attn(out: torch.Tensor, query: torch.Tensor, k_pool: torch.Tens
                                       ws_bytes, _stream(query))
     _lib.check(rc, lib)
     return out
+
+
+class PreparedDecode:
+    """``paged_decode_attn`` bound to fixed pools, block table, scales and head geometry.
+
+    The shape / dtype / device / contiguity checks of everything that does not change from step
+    to step run once, here; a call checks only the per-step tensors.  For callers that own their
+    pools and tables (one decode call per layer and token at small batch is bound by the host, not
+    by the GPU).  ``context_lens`` may be replaced per call by another contiguous int32 ``[B]``
+    tensor on the same device.
+    """
+
+    def __init__(self, k_pool: torch.Tensor, v_pool: torch.Tensor, block_table: torch.Tensor,
+                 context_lens: torch.Tensor, num_q_heads: int, q_dtype: torch.dtype, scale: float,
+                 k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
+                 partition_size: int = 0) -> None:
+        self.lib = _lib.load()
+        _req(k_pool.is_cuda, "tensors must live on a ROCm device (there is no CPU path)")
+        nb, hkv, bs, d = _check_pools(k_pool, v_pool)
+        B = block_table.shape[0]
+        _req(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1,
+             "block_table must be int32 [B, max_blocks], rows contiguous")
+        _req(context_lens.dtype == torch.int32 and context_lens.numel() == B and context_lens.is_contiguous(),
+             "context_lens must be contiguous int32 [B]")
+        _req(num_q_heads > 0 and num_q_heads % hkv == 0, f"{num_q_heads} query heads over {hkv} KV heads")
+        _dev(block_table, k_pool, "block_table")
+        _dev(context_lens, k_pool, "context_lens")
+        ks, vs = _check_scales(k_scale, v_scale, k_pool, hkv)
+        try:
+            qd = _DT[q_dtype]
+        except KeyError:
+            raise RuntimeError(f"query: unsupported dtype {q_dtype}")
+        self.device, self.q_dtype = k_pool.device, q_dtype
+        self.q_shape = (B, num_q_heads, d)
+        self.kv_shape = (B, hkv, d)
+        self.context_lens = context_lens
+        self.need = self.lib.aicomp_paged_decode_workspace_bytes(B, num_q_heads, hkv, d, bs, block_table.shape[1],
+                                                                 qd, _dt(k_pool, "pool"), partition_size)
+        # keep the tensors alive; everything below is what the C entry points take
+        self._keep = (k_pool, v_pool, block_table, ks, vs)
+        self._head = (k_pool.data_ptr(), v_pool.data_ptr(), block_table.data_ptr(), block_table.stride(0))
+        self._tail = (B, num_q_heads, hkv, d, bs, block_table.shape[1], nb, float(scale), qd,
+                      _dt(k_pool, "pool"), _ptr(ks), _ptr(vs), partition_size)
+
+    def __call__(self, out: torch.Tensor, query: torch.Tensor, new_key: Optional[torch.Tensor] = None,
+                 new_value: Optional[torch.Tensor] = None,
+                 context_lens: Optional[torch.Tensor] = None) -> torch.Tensor:
+        _req(query.shape == self.q_shape and out.shape == self.q_shape and query.dtype == self.q_dtype
+             and out.dtype == self.q_dtype and query.device == self.device and out.device == self.device
+             and query.is_contiguous() and out.is_contiguous(),
+             f"out/query must be contiguous {self.q_shape} {self.q_dtype} tensors on {self.device}")
+        ctx = self.context_lens if context_lens is None else context_lens
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        ws = _workspace(self.device, self.need, stream)
+        ws_ptr, ws_bytes = (None, 0) if ws is None else (ws.data_ptr(), ws.numel())
+        if new_key is None:
+            rc = self.lib.aicomp_paged_decode_attn(out.data_ptr(), query.data_ptr(), *self._head, ctx.data_ptr(),
+                                                   *self._tail, ws_ptr, ws_bytes, stream)
+        else:
+            _req(new_value is not None and new_key.shape == self.kv_shape and new_value.shape == self.kv_shape
+                 and new_key.dtype == self.q_dtype and new_value.dtype == self.q_dtype
+                 and new_key.device == self.device and new_value.device == self.device,
+                 f"new_key/new_value must both be {self.kv_shape} of the query dtype on {self.device}")
+            if new_key.stride(2) != 1 or new_key.stride() != new_value.stride():
+                new_key, new_value = new_key.contiguous(), new_value.contiguous()
+            rc = self.lib.aicomp_paged_decode_attn_append(
+                out.data_ptr(), query.data_ptr(), new_key.data_ptr(), new_value.data_ptr(),
+                new_key.stride(0), new_key.stride(1), *self._head, ctx.data_ptr(), *self._tail,
+                ws_ptr, ws_bytes, stream)
+        _lib.check(rc, self.lib)
+        return out
 
 
 def paged_prefill_attn(out: torch.Tensor, query: torch.Tensor, k_pool: torch.Tensor,

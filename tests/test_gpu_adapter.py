@@ -114,3 +114,37 @@ def test_adapter_llama32_1b_heads_bf16(device):
     _run_session(new, ref, B, hq, g, d, [77, 1, 1, 1, 1, 1], device, torch.bfloat16, 1e-2)
     assert new._group == 4 and new.cache_k.shape == (2 * 16, 8, 16, 64)
     new.disable()
+
+
+def test_adapter_batch_one_and_hf_style_views(device):
+    """Batch 1 (what the reference's examples run) with q/k/v arriving the way HF Llama builds them:
+    ``proj(x).view(B, n, H, D).transpose(1, 2)``, i.e. non-contiguous views; for batch 1 the
+    token-major reshape of such a tensor is itself a strided view."""
+    torch.manual_seed(3)
+    hq, g, d = 32, 4, 64
+    hkv = hq // g
+    new = akv.CachedScaledDotProductAttention(0, max_seq_len=128, dtype=torch.bfloat16)
+    ref = cref.ContiguousCachedAttention(0, 128)
+    new.enable(); ref.enable()
+    for n in [40, 1, 1, 1]:
+        qb = torch.randn(1, n, hq, d).to(torch.bfloat16)
+        kb = (torch.randn(1, n, hkv, d) * 0.5).to(torch.bfloat16)
+        vb = (torch.randn(1, n, hkv, d) * 0.5).to(torch.bfloat16)
+        q, k, v = (t.to(device).transpose(1, 2) for t in (qb, kb, vb))          # [1, H, n, D] views
+        ke, ve = k.repeat_interleave(g, 1), v.repeat_interleave(g, 1)
+        assert n == 1 or not q.is_contiguous()
+        got = new(q, ke, ve, is_causal=True)
+        want = ref(q.float().cpu(), ke.float().cpu(), ve.float().cpu(), attn_mask=None, is_causal=True)
+        assert got.shape == (1, hq, n, d)
+        err = (got.float().cpu() - want).abs()
+        assert bool(((err <= 1e-2) | (err <= 2e-2 * want.abs())).all()), f"n={n}: {err.max().item():.3e}"
+    # contiguous [1, H, n, D] inputs: the token-major reshape is then a strided view
+    new.clear(); ref.clear()
+    q = torch.randn(1, hq, 24, d).to(torch.bfloat16).to(device)
+    k = (torch.randn(1, hkv, 24, d) * 0.5).to(torch.bfloat16).to(device).repeat_interleave(g, 1)
+    v = (torch.randn(1, hkv, 24, d) * 0.5).to(torch.bfloat16).to(device).repeat_interleave(g, 1)
+    got = new(q, k, v, is_causal=True)
+    want = ref(q.float().cpu(), k.float().cpu(), v.float().cpu(), attn_mask=None, is_causal=True)
+    err = (got.float().cpu() - want).abs()
+    assert bool(((err <= 1e-2) | (err <= 2e-2 * want.abs())).all()), f"{err.max().item():.3e}"
+    new.disable()

@@ -354,3 +354,31 @@ def test_decode_head_dim_64_fused_append(device):
                           new_key=w.new_key, new_value=w.new_value)
     torch.cuda.synchronize()
     assert torch.equal(out, ref) and torch.equal(w.k_pool, kp) and torch.equal(w.v_pool, vp)
+
+
+@pytest.mark.parametrize("name", ["llama3_8b_decode", "llama3_70b_decode_fp8", "llama32_1b_decode", "decode_fp32_small"])
+def test_prepared_decode_equals_the_checked_call(device, name):
+    """The bound call (checks done once) launches exactly what ``paged_decode_attn`` launches: same
+    bits in the output and in the pools, with and without the fused append, and with a replaced
+    context-length tensor."""
+    w = workloads.make_workload("x", device=device, shape=small(name, batch=5))
+    t0 = int(w.cu_q_lens[w.num_prefill_seqs])
+    nk, nv = w.new_key[t0:].contiguous(), w.new_value[t0:].contiguous()
+    k1, v1, k2, v2 = w.k_pool.clone(), w.v_pool.clone(), w.k_pool.clone(), w.v_pool.clone()
+    call = ops.PreparedDecode(k2, v2, w.block_table, w.context_lens, w.query.shape[1], w.query.dtype, w.scale,
+                              w.k_scale, w.v_scale)
+    fused = w.query.dtype == nk.dtype
+    for step in range(3):
+        ctx = (w.context_lens - step).clamp_min(1).contiguous()
+        a = torch.full_like(w.query, float("nan"))
+        b = torch.full_like(w.query, float("nan"))
+        kw = dict(new_key=nk, new_value=nv) if fused and step != 1 else {}
+        ops.paged_decode_attn(a, w.query, k1, v1, w.block_table, ctx, w.scale, w.k_scale, w.v_scale, **kw)
+        call(b, w.query, kw.get("new_key"), kw.get("new_value"), context_lens=ctx)
+        torch.cuda.synchronize()
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), step
+        assert torch.equal(k1.view(torch.uint8), k2.view(torch.uint8)) and torch.equal(v1.view(torch.uint8), v2.view(torch.uint8))
+    with pytest.raises(RuntimeError):
+        call(torch.empty(5, 3, 7, device=device), w.query)
+    with pytest.raises(RuntimeError):
+        ops.PreparedDecode(k2, v2, w.block_table.to(torch.int64), w.context_lens, w.query.shape[1], w.query.dtype, w.scale)
