@@ -108,7 +108,7 @@ __device__ __forceinline__ void for_each_logit(const T* row, int begin, int end,
     int tail = begin;
     if (vec_ok) {
         const int n4 = (end - begin) / 4;              // begin is a multiple of 4 for every caller
-        constexpr int U = 8;                           // loads in flight per lane: the passes are latency bound
+        constexpr int U = 16;                          // loads in flight per lane: the passes are latency bound
         for (int j0 = rank; j0 < n4; j0 += U * nranks) {
             float a[U][4];
 #pragma unroll
@@ -163,8 +163,8 @@ __device__ __forceinline__ uint64_t wave_incl_scan64(uint64_t v, int lane) {
 
 // Shared state of the radix walks (one row)
 struct Shared {
-    unsigned long long mass[BINS];
-    unsigned int cnt[BINS];
+    alignas(16) unsigned long long mass[BINS];
+    alignas(16) unsigned int cnt[BINS];
     unsigned long long seg_mass[NW];
     unsigned int seg_tied[NW];
     float red_f[NW];
@@ -175,21 +175,33 @@ struct Shared {
     unsigned int sel_above_cnt;
     // candidates of the top-k fast path
     unsigned int n_list;
-    unsigned int list_key[LIST_CAP];
-    unsigned int list_idx[LIST_CAP];
-    unsigned long long list_w[LIST_CAP];
+    alignas(16) unsigned int list_key[LIST_CAP];
+    alignas(16) unsigned int list_idx[LIST_CAP];
+    alignas(16) unsigned long long list_w[LIST_CAP];
 };
 
 // Wave 0: walking the bins from the top, find the bin that holds the k-th element
 // (by count).  Returns digit and the count strictly above it.
 __device__ void pick_by_count(Shared& s, int nbins, unsigned int k, int lane) {
-    // lane owns bins [hi - 32*lane - 31, hi - 32*lane], i.e. lane 0 the top 32 bins
-    const int per = BINS / 64;
-    unsigned int local = 0;
-    for (int j = 0; j < per; ++j) {
-        const int b = nbins - 1 - (lane * per + j);
-        if (b >= 0) local += s.cnt[b];
+    // lane owns bins [hi - 32*lane - 31, hi - 32*lane], i.e. lane 0 the top 32 bins: read as eight
+    // 16-byte vectors (independent loads; a dependent chain of 32 LDS reads costs microseconds)
+    constexpr int per = BINS / 64;
+    const int top = nbins - 1 - lane * per;            // highest bin of this lane; nbins is a multiple of per
+    unsigned int c[per];                               // c[j] = count of bin top - j
+    if (top >= per - 1) {
+        const uint4* v = (const uint4*)&s.cnt[top - (per - 1)];
+#pragma unroll
+        for (int q = 0; q < per / 4; ++q) {
+            const uint4 x = v[q];
+            c[per - 1 - 4 * q] = x.x; c[per - 2 - 4 * q] = x.y; c[per - 3 - 4 * q] = x.z; c[per - 4 - 4 * q] = x.w;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < per; ++j) c[j] = 0;
     }
+    unsigned int local = 0;
+#pragma unroll
+    for (int j = 0; j < per; ++j) local += c[j];
     unsigned int incl = local;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -204,13 +216,15 @@ __device__ void pick_by_count(Shared& s, int nbins, unsigned int k, int lane) {
         unsigned int run = excl;
         int chosen = 0;
         unsigned int above = excl;
+        bool done = false;
+#pragma unroll
         for (int j = 0; j < per; ++j) {
-            const int b = nbins - 1 - (lane * per + j);
-            if (b < 0) break;
-            chosen = b;
-            above = run;
-            run += s.cnt[b];
-            if (run >= k) break;
+            if (!done && top - j >= 0) {
+                chosen = top - j;
+                above = run;
+                run += c[j];
+                done = run >= k;
+            }
         }
         s.sel_digit = (unsigned int)chosen;
         s.sel_above_cnt = above;
@@ -255,10 +269,13 @@ constexpr int WIDTHS[3] = {11, 11, 10};
 
 // Key of the k-th largest element of a source (all lanes call; `src(f)` runs f(index, value) over
 // the lane's share of the elements).  Three histogram rounds over digits of 11, 11 and 10 bits.
+// With fewer than three levels the result is the lower edge of the bin that holds the k-th largest
+// element at that resolution: a lower bound of its key.
 template <typename Src>
-__device__ __forceinline__ uint32_t select_kth(Shared& s, Src src, unsigned int k, int tid, int lane, int wave) {
+__device__ __forceinline__ uint32_t select_kth(Shared& s, Src src, unsigned int k, int tid, int lane, int wave,
+                                               int levels = 3) {
     uint32_t prefix = 0, pmask = 0;
-    for (int lvl = 0; lvl < 3; ++lvl) {
+    for (int lvl = 0; lvl < levels; ++lvl) {
         const int nb = 1 << WIDTHS[lvl];
         const int sh = SHIFTS[lvl];
         __syncthreads();
@@ -350,37 +367,59 @@ sample_kernel(SampleParams p) {
     const int V = p.vocab;
     const float temp = p.greedy ? 1.f : p.temperature;
 
-    // ---------------------------------------------------------------- 1. maximum / argmax
+    // ---------------------------------------------------------------- 1. maximum (greedy: argmax)
     // On the raw logits: dividing by a positive temperature keeps the order, so the maximum of
-    // the scaled row is the scaled maximum and no division is needed in this pass.
-    float best = -INFINITY;
-    int best_i = 0x7fffffff;
+    // the scaled row is the scaled maximum and no division is needed in this pass.  Sampling only
+    // needs the value (one v_max per element); the index is found by a second pass in the rare
+    // case that asks for it (greedy decoding, or a row without any finite mass).
     const bool vec_ok = ((uintptr_t)row % 16) == 0;
-    for_each_logit<T>(row, 0, V, 1.f, tid, NT, vec_ok, [&](int i, float x) {
-        if (x > best) { best = x; best_i = i; }       // lowest index wins ties within a lane (ascending i)
-    });
-    const float lane_best = best;                     // raw maximum of this lane's share of the row
+    auto block_argmax = [&]() -> int {
+        float best = -INFINITY;
+        int best_i = 0x7fffffff;
+        for_each_logit<T>(row, 0, V, 1.f, tid, NT, vec_ok, [&](int i, float x) {
+            if (x > best) { best = x; best_i = i; }       // lowest index wins ties within a lane (ascending i)
+        });
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const float ob = __shfl_xor(best, o);
-        const int oi = __shfl_xor(best_i, o);
-        if (ob > best || (ob == best && oi < best_i)) { best = ob; best_i = oi; }
-    }
-    if (lane == 0) { s.red_f[wave] = best; s.red_i[wave] = best_i; }
-    __syncthreads();
-    best = s.red_f[0]; best_i = s.red_i[0];
-    for (int w = 1; w < NW; ++w) {
-        const float ob = s.red_f[w];
-        const int oi = s.red_i[w];
-        if (ob > best || (ob == best && oi < best_i)) { best = ob; best_i = oi; }
-    }
-    const float m = apply_temperature<T>(best, temp);
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o);
+            const int oi = __shfl_xor(best_i, o);
+            if (ob > best || (ob == best && oi < best_i)) { best = ob; best_i = oi; }
+        }
+        __syncthreads();
+        if (lane == 0) { s.red_f[wave] = best; s.red_i[wave] = best_i; }
+        __syncthreads();
+        best = s.red_f[0]; best_i = s.red_i[0];
+        for (int w = 1; w < NW; ++w) {
+            const float ob = s.red_f[w];
+            const int oi = s.red_i[w];
+            if (ob > best || (ob == best && oi < best_i)) { best = ob; best_i = oi; }
+        }
+        return best_i == 0x7fffffff ? 0 : best_i;
+    };
     if (p.greedy) {
-        if (tid == 0) p.out[row_idx] = best_i == 0x7fffffff ? 0 : best_i;
+        const int best_i = block_argmax();
+        if (tid == 0) p.out[row_idx] = best_i;
         if (p.probs_out)
             for (int i = tid; i < V; i += NT) p.probs_out[(int64_t)row_idx * V + i] = i == best_i ? 1.f : 0.f;
         return;
     }
+    // a row without finite mass (all -inf, NaN): the argmax, and an all-zero distribution
+    auto no_mass = [&]() {
+        const int best_i = block_argmax();
+        if (tid == 0) p.out[row_idx] = best_i;
+        if (p.probs_out)
+            for (int i = tid; i < V; i += NT) p.probs_out[(int64_t)row_idx * V + i] = 0.f;
+    };
+    float lane_best = -INFINITY;                      // raw maximum of this lane's share of the row
+    for_each_logit<T>(row, 0, V, 1.f, tid, NT, vec_ok, [&](int, float x) { lane_best = fmaxf(lane_best, x); });
+    float best = lane_best;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) best = fmaxf(best, __shfl_xor(best, o));
+    if (lane == 0) s.red_f[wave] = best;
+    __syncthreads();
+    best = s.red_f[0];
+    for (int w = 1; w < NW; ++w) best = fmaxf(best, s.red_f[w]);
+    const float m = apply_temperature<T>(best, temp);
 
     auto over_row = [&](auto f) { for_each_logit<T>(row, 0, V, temp, tid, NT, vec_ok, f); };
     auto over_list = [&](auto f) {
@@ -401,14 +440,20 @@ sample_kernel(SampleParams p) {
     const bool topk_on = p.top_k > 0 && p.top_k < V;
     if (topk_on && p.top_k <= NT && temp <= LIST_MAX_TEMPERATURE) {
         auto over_lane_max = [&](auto f) { f(tid, lane_best); };
-        const uint32_t key_l = select_kth(s, over_lane_max, (unsigned int)p.top_k, tid, lane, wave);
+        // two digit levels (22 of 32 key bits): a bound 2^-13 relative below the k-th largest maximum
+        // lets in a few more candidates and saves a histogram round
+        const uint32_t key_l = select_kth(s, over_lane_max, (unsigned int)p.top_k, tid, lane, wave, 2);
         const uint32_t key_ls = order_key(apply_temperature<T>(key_value(key_l), temp));
         const uint32_t slack = LIST_SLACK * (sizeof(T) == 2 ? 0x10000u : 1u);     // bf16 values are 2^16 keys apart
         const uint32_t key_lo = key_l > slack ? key_l - slack : 0u;
         if (tid == 0) s.n_list = 0;
         __syncthreads();
+        // prefilter on the raw float, one compare per element.  It lets through whatever the key
+        // order would (plus -0.0 next to +0.0, and everything when the bound is below -inf, whose
+        // key decodes to a NaN); the exact test on the scaled key follows.
+        const float raw_lo = key_value(key_lo);
         for_each_logit<T>(row, 0, V, 1.f, tid, NT, vec_ok, [&](int i, float x) {
-            if (order_key(x) >= key_lo) {
+            if (!(x < raw_lo)) {
                 const uint32_t key = order_key(apply_temperature<T>(x, temp));
                 if (key >= key_ls) {
                     const unsigned int j = atomicAdd(&s.n_list, 1u);
@@ -418,6 +463,87 @@ sample_kernel(SampleParams p) {
         });
         __syncthreads();
         use_list = s.n_list <= LIST_CAP;
+    }
+    if (use_list && s.n_list <= NT && s.n_list >= (unsigned int)p.top_k) {
+        // ------------------------------------------------------------ 2a. at most one candidate per lane
+        // (the usual case: about k of them).  No histograms: every lane ranks its candidate in the
+        // descending order a stable sort would give (key, then index), the lane of rank k-1 holds
+        // the k-th largest key, the mass that precedes a candidate in that order decides the
+        // nucleus, and the draw walks the kept candidates in index order.  Plain loops over the
+        // list in LDS, exact 64-bit sums.
+        const int n = (int)s.n_list;
+        const bool mine = tid < n;
+        const uint32_t key = mine ? s.list_key[tid] : 0u;
+        const unsigned int idx = mine ? s.list_idx[tid] : 0xffffffffu;
+        // the loops below read the list eight entries at a time (independent LDS reads; entries past
+        // n are inside the arrays and masked out)
+        unsigned int rank = 0;
+        if (mine)
+            for (int i0 = 0; i0 < n; i0 += 8) {
+                uint32_t kk[8], ii[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) { kk[u] = s.list_key[i0 + u]; ii[u] = s.list_idx[i0 + u]; }
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    rank += (i0 + u < n) && ((kk[u] > key) || (kk[u] == key && ii[u] < idx));
+            }
+        if (mine && rank == (unsigned int)p.top_k - 1u) s.sel_digit = key;     // ranks are a permutation: one writer
+        __syncthreads();
+        const uint32_t kth = s.sel_digit;
+        uint64_t w = (mine && key >= kth) ? weight_of(key_value(key), m) : 0;   // ties at the k-th value all stay
+        if (mine) { s.cnt[tid] = rank; s.list_w[tid] = w; }
+        unsigned long long z = wave_sum64(w);
+        if (lane == 0) s.seg_mass[wave] = z;
+        __syncthreads();
+        z = 0;
+        for (int wv = 0; wv < NW; ++wv) z += s.seg_mass[wv];
+        if (p.top_p < 1.f) {
+            // an entry stays while the mass before it (in sorted order) is at most top_p of the total
+            const unsigned long long limit = (unsigned long long)((double)fmaxf(p.top_p, 0.f) * (double)z);
+            unsigned long long before = 0;
+            if (w)
+                for (int i0 = 0; i0 < n; i0 += 8) {
+                    uint32_t rr[8];
+                    unsigned long long ww[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) { rr[u] = s.cnt[i0 + u]; ww[u] = s.list_w[i0 + u]; }
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) before += (i0 + u < n && rr[u] < rank) ? ww[u] : 0ull;
+                }
+            if (before > limit) w = 0;
+            __syncthreads();                       // every lane has read the unfiltered weights
+            if (mine) s.list_w[tid] = w;
+            z = wave_sum64(w);
+            if (lane == 0) s.seg_mass[wave] = z;
+            __syncthreads();
+            z = 0;
+            for (int wv = 0; wv < NW; ++wv) z += s.seg_mass[wv];
+        }
+        if (z == 0) {                                  // non-finite logits: fall back to the argmax
+            no_mass();
+            return;
+        }
+        unsigned long long target = (unsigned long long)((double)p.uniforms[row_idx] * (double)z);
+        if (target >= z) target = z - 1;
+        if (p.probs_out) {
+            for (int i = tid; i < V; i += NT) p.probs_out[(int64_t)row_idx * V + i] = 0.f;
+            __syncthreads();
+        }
+        if (w) {
+            unsigned long long before = 0;             // kept mass at lower indices
+            for (int i0 = 0; i0 < n; i0 += 8) {
+                uint32_t ii[8];
+                unsigned long long ww[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) { ii[u] = s.list_idx[i0 + u]; ww[u] = s.list_w[i0 + u]; }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) before += (i0 + u < n && ii[u] < idx) ? ww[u] : 0ull;
+            }
+            if (before <= target && target < before + w) p.out[row_idx] = idx;
+            const double inv_z = 1.0 / (double)z;
+            if (p.probs_out) p.probs_out[(int64_t)row_idx * V + idx] = (float)((double)w * inv_z);
+        }
+        return;
     }
     if (topk_on)
         key_k = use_list ? select_kth(s, over_list, (unsigned int)p.top_k, tid, lane, wave)
@@ -462,9 +588,7 @@ sample_kernel(SampleParams p) {
         unsigned long long z2 = 0;
         for (int w = 0; w < NW; ++w) z2 += s.seg_mass[w];
         if (z2 == 0) {                                 // non-finite logits: fall back to the argmax
-            if (tid == 0) p.out[row_idx] = best_i == 0x7fffffff ? 0 : best_i;
-            if (p.probs_out)
-                for (int i = tid; i < V; i += NT) p.probs_out[(int64_t)row_idx * V + i] = 0.f;
+            no_mass();
             return;
         }
         unsigned long long target = (unsigned long long)((double)p.uniforms[row_idx] * (double)z2);
@@ -515,9 +639,7 @@ sample_kernel(SampleParams p) {
         tied_base += nt;
     }
     if (z2 == 0) {                                 // no mass at all (non-finite logits): fall back to the argmax
-        if (tid == 0) p.out[row_idx] = best_i == 0x7fffffff ? 0 : best_i;
-        if (p.probs_out)
-            for (int i = tid; i < V; i += NT) p.probs_out[(int64_t)row_idx * V + i] = 0.f;
+        no_mass();
         return;
     }
     unsigned long long target = (unsigned long long)((double)p.uniforms[row_idx] * (double)z2);

@@ -146,3 +146,23 @@ def test_rejects_bad_arguments(device):
         ops.sample_tokens(x, uniforms=torch.rand(3, device=device))
     with pytest.raises(RuntimeError):
         ops.sample_tokens(x.t())
+
+
+def test_masked_vocabulary(device):
+    """Rows where most of the vocabulary is masked with -inf, the way a constrained decoder hands
+    them over: fewer finite logits than top_k, exactly top_k, many more; -inf entries get no mass.
+    A row without any finite logit returns the argmax convention (index 0) and an all-zero row."""
+    rng = np.random.default_rng(9)
+    V = 6000
+    x = np.full((5, V), -np.inf, dtype=np.float32)
+    for b, n_finite in enumerate([1, 10, 50, 51, 3000]):
+        idx = rng.choice(V, n_finite, replace=False)
+        x[b, idx] = (rng.standard_normal(n_finite) * 2).astype(np.float32)
+    for temperature, top_k, top_p in [(0.8, 50, 0.9), (1.0, 50, 1.0), (1.0, 0, 0.9), (1.0, 0, 1.0), (1.3, 2000, 0.5)]:
+        tok, probs = check_rows(device, x, temperature, top_k, top_p)
+        assert np.all(probs[~np.isfinite(x)] == 0)
+    dead = torch.full((2, 300), float("-inf"), device=device)
+    tok, probs = ops.sample_tokens(dead, 0.8, 50, 0.9, True, torch.tensor([0.3, 0.9], device=device), return_probs=True)
+    assert tok.tolist() == [0, 0] and float(probs.abs().sum()) == 0.0
+    tok = ops.sample_tokens(dead, do_sample=False)
+    assert tok.tolist() == [0, 0]
