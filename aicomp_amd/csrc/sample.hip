@@ -130,10 +130,17 @@ __device__ __forceinline__ void for_each_logit(const T* row, int begin, int end,
     for (int i = tail + rank; i < end; i += nranks) f(i, scaled_logit<T>(row, i, temperature));
 }
 
-// 2^-40 fixed-point weight exp(x - m) of a logit
+// 2^-40 fixed-point weight exp(x - m) of a logit (x <= m, so the weight is in [0, 1]): the hardware
+// exponential, then the two 32-bit halves of w * 2^40 from two float -> uint32 conversions (a
+// float -> uint64 conversion is a long instruction sequence, and this runs once per logit in the
+// full-row passes).  A NaN logit gets weight 0.
 __device__ __forceinline__ uint64_t weight_of(float x, float m) {
-    const float w = exp2f((x - m) * LOG2E);
-    return (uint64_t)(w * W_ONE + 0.5f);
+    const float w = __builtin_amdgcn_exp2f((x - m) * LOG2E);
+    const float s8 = w * 256.f;                                  // exact scaling, [0, 256]
+    const float hi_f = floorf(s8);
+    const uint32_t hi = (uint32_t)hi_f;                          // w * 2^8, integer part
+    const uint32_t lo = (uint32_t)((s8 - hi_f) * 4294967296.f);  // fraction * 2^32 (the difference is exact)
+    return ((uint64_t)hi << 32) | lo;
 }
 
 __device__ __forceinline__ uint64_t shfl64(uint64_t v, int src) {
