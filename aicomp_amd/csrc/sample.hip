@@ -311,10 +311,14 @@ struct Nucleus {
 // Nucleus threshold over the elements with key >= key_k: the same radix walk on mass histograms.
 template <typename Src>
 __device__ __forceinline__ Nucleus nucleus_threshold(Shared& s, Src src, uint32_t key_k, float m, float top_p,
-                                                     int tid, int lane, int wave) {
-    uint32_t prefix = 0, pmask = 0;
-    unsigned long long limit = 0;
-    for (int lvl = 0; lvl < 3; ++lvl) {
+                                                     int tid, int lane, int wave, int first_level = 0,
+                                                     uint32_t prefix0 = 0, uint32_t pmask0 = 0,
+                                                     unsigned long long limit0 = 0) {
+    // first_level > 0: the caller has already walked the upper digit levels (prefix, mask and what is
+    // left of the mass limit below the bins above the chosen one)
+    uint32_t prefix = prefix0, pmask = pmask0;
+    unsigned long long limit = limit0;
+    for (int lvl = first_level; lvl < 3; ++lvl) {
         const int nb = 1 << WIDTHS[lvl];
         const int sh = SHIFTS[lvl];
         __syncthreads();
@@ -444,6 +448,9 @@ sample_kernel(SampleParams p) {
     // (masses of equal values) takes the full-row walk.
     uint32_t key_k = 0;                          // keep keys >= key_k
     bool use_list = false;
+    int nuc_first = 0;                           // nucleus walk already done down to this digit level (no top-k) ...
+    uint32_t nuc_prefix = 0, nuc_pmask = 0;      // ... with this key prefix ...
+    unsigned long long nuc_limit = 0;            // ... and this much of the mass limit left
     const bool topk_on = p.top_k > 0 && p.top_k < V;
     if (topk_on && p.top_k <= NT && temp <= LIST_MAX_TEMPERATURE) {
         auto over_lane_max = [&](auto f) { f(tid, lane_best); };
@@ -471,13 +478,13 @@ sample_kernel(SampleParams p) {
         __syncthreads();
         use_list = s.n_list <= LIST_CAP;
     }
-    if (use_list && s.n_list <= NT && s.n_list >= (unsigned int)p.top_k) {
-        // ------------------------------------------------------------ 2a. at most one candidate per lane
-        // (the usual case: about k of them).  No histograms: every lane ranks its candidate in the
-        // descending order a stable sort would give (key, then index), the lane of rank k-1 holds
-        // the k-th largest key, the mass that precedes a candidate in that order decides the
-        // nucleus, and the draw walks the kept candidates in index order.  Plain loops over the
-        // list in LDS, exact 64-bit sums.
+    // ---------------------------------------------------------------- at most one candidate per lane
+    // No histograms: every lane ranks its candidate in the descending order a stable sort would give
+    // (key, then index); with top-k the lane of rank k-1 holds the k-th largest key; the mass that
+    // precedes a candidate in that order decides the nucleus; the draw walks the kept candidates in
+    // index order.  Plain loops over the list in LDS, exact 64-bit sums.  Without top-k the list is
+    // everything above a cut of the whole row and z_row the mass of the whole row.
+    auto draw_from_small_list = [&](bool has_topk, unsigned long long z_row) {
         const int n = (int)s.n_list;
         const bool mine = tid < n;
         const uint32_t key = mine ? s.list_key[tid] : 0u;
@@ -494,9 +501,9 @@ sample_kernel(SampleParams p) {
                 for (int u = 0; u < 8; ++u)
                     rank += (i0 + u < n) && ((kk[u] > key) || (kk[u] == key && ii[u] < idx));
             }
-        if (mine && rank == (unsigned int)p.top_k - 1u) s.sel_digit = key;     // ranks are a permutation: one writer
+        if (has_topk && mine && rank == (unsigned int)p.top_k - 1u) s.sel_digit = key;   // ranks are a permutation: one writer
         __syncthreads();
-        const uint32_t kth = s.sel_digit;
+        const uint32_t kth = has_topk ? s.sel_digit : 0u;
         uint64_t w = (mine && key >= kth) ? weight_of(key_value(key), m) : 0;   // ties at the k-th value all stay
         if (mine) { s.cnt[tid] = rank; s.list_w[tid] = w; }
         unsigned long long z = wave_sum64(w);
@@ -506,7 +513,8 @@ sample_kernel(SampleParams p) {
         for (int wv = 0; wv < NW; ++wv) z += s.seg_mass[wv];
         if (p.top_p < 1.f) {
             // an entry stays while the mass before it (in sorted order) is at most top_p of the total
-            const unsigned long long limit = (unsigned long long)((double)fmaxf(p.top_p, 0.f) * (double)z);
+            // (of the row's total when the list is a cut of the whole row rather than its top k)
+            const unsigned long long limit = (unsigned long long)((double)fmaxf(p.top_p, 0.f) * (double)(has_topk ? z : z_row));
             unsigned long long before = 0;
             if (w)
                 for (int i0 = 0; i0 < n; i0 += 8) {
@@ -550,7 +558,86 @@ sample_kernel(SampleParams p) {
             const double inv_z = 1.0 / (double)z;
             if (p.probs_out) p.probs_out[(int64_t)row_idx * V + idx] = (float)((double)w * inv_z);
         }
+    };
+    if (use_list && s.n_list <= NT && s.n_list >= (unsigned int)p.top_k) {
+        draw_from_small_list(true, 0ull);
         return;
+    }
+
+    // ---------------------------------------------------------------- 2b. nucleus without top-k
+    // One pass gives the exact mass of the row and, for the logits within NUCLEUS_SPAN of the
+    // maximum only (the rest cannot hold the threshold unless the row is very flat, and would cost
+    // an LDS atomic each), a first-level mass histogram.  If the walk finds the threshold bin inside
+    // that region, everything from that bin up is collected and, when it fits one candidate per
+    // lane, handled like a top-k list.  Otherwise the full-row walk below runs.
+    if (!topk_on && p.top_p < 1.f) {
+        constexpr float NUCLEUS_SPAN = 12.f;
+        const float cut_f = m - NUCLEUS_SPAN;
+        const int nb0 = 1 << WIDTHS[0];
+        for (int b2 = tid; b2 < BINS; b2 += NT) { s.mass[b2] = 0; s.cnt[b2] = 0; }
+        if (tid == 0) s.n_list = 0;
+        __syncthreads();
+        unsigned long long zacc = 0;
+        over_row([&](int, float x) {
+            const uint64_t w = weight_of(x, m);
+            zacc += w;
+            if (x >= cut_f) {
+                const int b2 = (int)(order_key(x) >> SHIFTS[0]) & (nb0 - 1);
+                atomicAdd(&s.mass[b2], (unsigned long long)w);
+                atomicAdd(&s.cnt[b2], 1u);
+            }
+        });
+        zacc = wave_sum64(zacc);
+        if (lane == 0) s.seg_mass[wave] = zacc;
+        __syncthreads();
+        unsigned long long z_row = 0;
+        for (int wv = 0; wv < NW; ++wv) z_row += s.seg_mass[wv];
+        if (z_row == 0) {
+            no_mass();
+            return;
+        }
+        const unsigned long long limit = (unsigned long long)((double)fmaxf(p.top_p, 0.f) * (double)z_row);
+        if (wave == 0) pick_by_mass(s, nb0, limit, lane);
+        __syncthreads();
+        const uint32_t d0 = s.sel_digit;
+        if (d0 > (order_key(cut_f) >> SHIFTS[0])) {               // the whole bin lies inside the histogrammed region
+            // candidates from that bin up
+            unsigned int c = (tid >= (int)d0 ? s.cnt[tid] : 0u) + (tid + NT >= (int)d0 ? s.cnt[tid + NT] : 0u);
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o);
+            if (lane == 0) s.seg_tied[wave] = c;
+            __syncthreads();
+            unsigned int n_est = 0;
+            for (int wv = 0; wv < NW; ++wv) n_est += s.seg_tied[wv];
+            const uint32_t key_lo_s = d0 << SHIFTS[0];
+            if (n_est <= (unsigned int)NT) {
+                // raw prefilter: the scaled bound times the temperature, lowered by more than the division
+                // (and, for bf16 rows, the rounding of the quotient) can move a value
+                const float t_raw = key_value(key_lo_s) * temp;
+                const float raw_lo = temp == 1.f ? key_value(key_lo_s)
+                                                 : t_raw - fabsf(t_raw) * (sizeof(T) == 2 ? 0.0078125f : 9.5367431640625e-7f);
+                for_each_logit<T>(row, 0, V, 1.f, tid, NT, vec_ok, [&](int i, float x) {
+                    if (!(x < raw_lo)) {
+                        const uint32_t key = order_key(apply_temperature<T>(x, temp));
+                        if (key >= key_lo_s) {
+                            const unsigned int j = atomicAdd(&s.n_list, 1u);
+                            if (j < LIST_CAP) { s.list_key[j] = key; s.list_idx[j] = (unsigned int)i; }
+                        }
+                    }
+                });
+                __syncthreads();
+                if (s.n_list <= NT) {
+                    draw_from_small_list(false, z_row);
+                    return;
+                }
+            }
+            // too many for a list: the full-row walk continues below from the second digit level
+            nuc_first = 1;
+            nuc_prefix = key_lo_s;
+            nuc_pmask = (uint32_t)(nb0 - 1) << SHIFTS[0];
+            nuc_limit = limit - s.sel_above_mass;
+        }
+        __syncthreads();
     }
     if (topk_on)
         key_k = use_list ? select_kth(s, over_list, (unsigned int)p.top_k, tid, lane, wave)
@@ -561,7 +648,8 @@ sample_kernel(SampleParams p) {
     nu.key_t = key_k; nu.tie_keep = 0xffffffffu; nu.tie_rule = false;
     if (p.top_p < 1.f)
         nu = use_list ? nucleus_threshold(s, over_list, key_k, m, p.top_p, tid, lane, wave)
-                      : nucleus_threshold(s, over_row, key_k, m, p.top_p, tid, lane, wave);
+                      : nucleus_threshold(s, over_row, key_k, m, p.top_p, tid, lane, wave, nuc_first, nuc_prefix,
+                                          nuc_pmask, nuc_limit);
     const uint32_t key_t = nu.key_t;
     const unsigned int tie_keep = nu.tie_keep;
     const bool tie_rule = nu.tie_rule;
@@ -581,7 +669,13 @@ sample_kernel(SampleParams p) {
             if (tie_rule ? key > key_t : key >= key_t) w = weight_of(key_value(key), m);
             else if (tie_rule && key == key_t) {
                 unsigned int rank = 0;
-                for (int i = 0; i < n; ++i) rank += s.list_key[i] == key_t && s.list_idx[i] < idx;
+                for (int i0 = 0; i0 < n; i0 += 8) {
+                    uint32_t kk[8], ii[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) { kk[u] = s.list_key[min(i0 + u, n - 1)]; ii[u] = s.list_idx[min(i0 + u, n - 1)]; }
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) rank += i0 + u < n && kk[u] == key_t && ii[u] < idx;
+                }
                 if (rank < tie_keep) w = w_tie;
             }
             s.list_w[j] = w;
@@ -605,14 +699,54 @@ sample_kernel(SampleParams p) {
             __syncthreads();
         }
         const double inv_z = 1.0 / (double)z2;
+        if (p.probs_out)
+            for (int j = tid; j < n; j += NT) {
+                const uint64_t w = s.list_w[j];
+                if (w) p.probs_out[(int64_t)row_idx * V + s.list_idx[j]] = (float)((double)w * inv_z);
+            }
+        // The draw in index order without comparing every pair of entries: kept mass per bucket of
+        // consecutive indices (one bucket per lane), a scan over the buckets to find the one that
+        // holds the target, then the few entries of that bucket among themselves.
+        int sh = 0;
+        while (((V - 1) >> sh) >= NT) ++sh;
+        __syncthreads();
+        s.mass[tid] = 0;                               // NT <= BINS buckets
+        if (tid == 0) s.sel_above_cnt = 0;
+        __syncthreads();
         for (int j = tid; j < n; j += NT) {
             const uint64_t w = s.list_w[j];
-            if (!w) continue;
+            if (w) atomicAdd(&s.mass[s.list_idx[j] >> sh], (unsigned long long)w);
+        }
+        __syncthreads();
+        const unsigned long long mine_b = s.mass[tid];
+        unsigned long long incl = wave_incl_scan64(mine_b, lane);
+        if (lane == 63) s.seg_mass[wave] = incl;
+        __syncthreads();
+        unsigned long long base = 0;
+        for (int w = 0; w < wave; ++w) base += s.seg_mass[w];
+        incl += base;
+        if (mine_b && incl - mine_b <= target && target < incl) {      // exactly one bucket
+            s.sel_digit = (unsigned int)tid;
+            s.sel_above_mass = incl - mine_b;
+        }
+        __syncthreads();
+        const unsigned int bucket = s.sel_digit;
+        const unsigned long long bucket_base = s.sel_above_mass;
+        // the list positions of that bucket's entries go to the key array (the keys are no longer needed)
+        for (int j = tid; j < n; j += NT)
+            if (s.list_w[j] && (s.list_idx[j] >> sh) == bucket) s.list_key[atomicAdd(&s.sel_above_cnt, 1u)] = (unsigned int)j;
+        __syncthreads();
+        const int nb = (int)s.sel_above_cnt;           // at most n
+        for (int a = tid; a < nb; a += NT) {
+            const int j = (int)s.list_key[a];
             const unsigned int idx = s.list_idx[j];
-            unsigned long long before = 0;
-            for (int i = 0; i < n; ++i) before += s.list_idx[i] < idx ? s.list_w[i] : 0ull;
+            const unsigned long long w = s.list_w[j];
+            unsigned long long before = bucket_base;
+            for (int b = 0; b < nb; ++b) {
+                const int i = (int)s.list_key[b];
+                before += s.list_idx[i] < idx ? s.list_w[i] : 0ull;
+            }
             if (before <= target && target < before + w) p.out[row_idx] = idx;
-            if (p.probs_out) p.probs_out[(int64_t)row_idx * V + idx] = (float)((double)w * inv_z);
         }
         return;
     }

@@ -166,3 +166,23 @@ def test_masked_vocabulary(device):
     assert tok.tolist() == [0, 0] and float(probs.abs().sum()) == 0.0
     tok = ops.sample_tokens(dead, do_sample=False)
     assert tok.tolist() == [0, 0]
+
+
+def test_nucleus_without_top_k_routes(device):
+    """top-p without top-k takes one of three routes: a short candidate list above a cut near the
+    maximum (peaked rows), the full-row walk resumed below the first digit level (a nucleus of
+    thousands), or the complete full-row walk (the threshold lies far below the maximum)."""
+    rng = np.random.default_rng(11)
+    V = 40000
+    peaked = (rng.standard_normal((3, V)) * 2).astype(np.float32)
+    for b in range(3):
+        peaked[b, rng.choice(V, 25, replace=False)] = 12 + rng.standard_normal(25).astype(np.float32) * 3
+    broad = (rng.standard_normal((3, V)) * 3.5).astype(np.float32)
+    far = np.zeros((2, V), dtype=np.float32)
+    far[:, 17] = 13.0                                   # one strong token, the rest tied 13 below it
+    far[1, 5000:5100] = 2.0
+    for x in (peaked, broad, far):
+        for temperature, top_p in [(1.0, 0.9), (0.8, 0.5), (1.3, 0.97)]:
+            check_rows(device, x, temperature, 0, top_p)
+    check_rows(device, peaked, 0.7, 0, 0.9, dtype=torch.bfloat16)
+    check_rows(device, broad, 0.7, 0, 0.9, dtype=torch.bfloat16)
