@@ -253,7 +253,15 @@ static int decode_impl(void* out, const void* query, const void* new_key, const 
         }
         return launch_decode_streamk(a, workspace);
     }
-    if (fused) {
+    // the grid-scheduled matrix-core kernel appends the new rows itself under the same conditions
+    const bool mfma = decode_mfma_supported(a);
+    const bool in_kernel = fused && mfma && q_dtype == AICOMP_KV_BF16 && kv_token_stride % 8 == 0 &&
+                           kv_head_stride % 8 == 0 && (uintptr_t)new_key % 16 == 0 &&
+                           (uintptr_t)new_value % 16 == 0;
+    if (in_kernel) {
+        a.new_key = new_key; a.new_value = new_value;
+        a.new_token_stride = kv_token_stride; a.new_head_stride = kv_head_stride;
+    } else if (fused) {
         rc = launch_kv_append_last(new_key, new_value, kv_token_stride, kv_head_stride, k_pool, v_pool,
                                    block_table, block_table_stride, context_lens, batch, num_kv_heads,
                                    head_dim, block_size, max_blocks_per_seq, num_blocks, q_dtype,
@@ -269,7 +277,7 @@ static int decode_impl(void* out, const void* query, const void* new_key, const 
                        "%s: workspace must be 16-byte aligned", who);
         a.ws = split_workspace_view(workspace, a.rows, a.hq, a.hkv, a.d, a.num_parts);
     }
-    if (decode_mfma_supported(a)) return launch_decode_mfma(a);
+    if (mfma) return launch_decode_mfma(a);
     return launch_decode_generic(a);
 }
 

@@ -63,8 +63,8 @@ constexpr int SK_MAX_WAVES = 4096;     // balanced schedule: at most 1024 workgr
 struct MfmaParams {
     void* out;
     const void* query;
-    const void* k_pool;
-    const void* v_pool;
+    void* k_pool;
+    void* v_pool;
     const int32_t* block_table;
     int64_t block_table_stride;
     const int32_t* context_lens;
@@ -76,6 +76,10 @@ struct MfmaParams {
     int partition_size, num_parts;
     float* ws_acc;
     float* ws_ml;
+    // fused append (optional): row b of new_key / new_value is token context_lens[b]-1
+    const bf16_t* new_key;
+    const bf16_t* new_value;
+    int64_t new_token_stride, new_head_stride;     // elements
 };
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
@@ -277,6 +281,59 @@ __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, T
         st.O[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, af[j]), pf, st.O[j], 0, 0, 0);
 }
 
+// 8 floats -> 8 e4m3 codes: clamp(x / scale, +-448), round to nearest even
+__device__ __forceinline__ uint2 quant8_fp8(const uint4& bf, float scale) {
+    const uint32_t w[4] = {bf.x, bf.y, bf.z, bf.w};
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = fminf(fmaxf(__uint_as_float(w[i] << 16) / scale, -448.f), 448.f);
+        f[2 * i + 1] = fminf(fmaxf(__uint_as_float(w[i] & 0xffff0000u) / scale, -448.f), 448.f);
+    }
+    int lo = 0, hi = 0;
+    lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], lo, false);
+    lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
+    hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], hi, false);
+    hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
+    return make_uint2((uint32_t)lo, (uint32_t)hi);
+}
+
+// Fused append for the grid-scheduled kernel: the tile that holds the sequence's newest token
+// (context_lens - 1) takes its K/V row from new_key / new_value instead of what was loaded from
+// the pool, and writes it to the pool (the append itself).  No other wave of the launch reads
+// that token.  A tile row is one token (16 lanes of 8 elements), or with PAIR half a row (8 lanes).
+template <bool FP8, bool PAIR>
+__device__ __forceinline__ void inject_new_row_grid(TileRegs<FP8>& kr, TileRegs<FP8>& vr, const MfmaParams& p,
+                                                    int seq, int kvh, int lane, int tile_start, int len,
+                                                    const int64_t (&bb)[4]) {
+    constexpr int DQ = PAIR ? 64 : D;
+    const int tau = len - 1 - tile_start;              // token within the tile, wave-uniform
+    const int blk_i = tau >> 4, tb = tau & 15;         // block of the tile, token within the block
+    const int c = PAIR ? (lane & 7) : (lane & 15);     // 8-element chunk of the new row this lane holds
+    // register slot and lanes of that token: load i of lane l is row 4i + l/16 (chunk l%16) of the tile
+    const int row = PAIR ? (tau >> 1) : tau;
+    const bool mine = (lane >> 4) == (row & 3) && (!PAIR || ((lane >> 3) & 1) == (tau & 1));
+    const int slot = row >> 2;
+    const int64_t src = (int64_t)seq * p.new_token_stride + (int64_t)kvh * p.new_head_stride + 8 * c;
+    const uint4 nk = *(const uint4*)(p.new_key + src);
+    const uint4 nv = *(const uint4*)(p.new_value + src);
+    const int64_t blk = bb[blk_i];
+    const int64_t dst = ((blk * p.hkv + kvh) * BS + tb) * (DQ / 8) + c;        // 8-element chunks
+    if constexpr (FP8) {
+        const uint2 ck = quant8_fp8(nk, p.k_scale[kvh]);
+        const uint2 cv = quant8_fp8(nv, p.v_scale[kvh]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (mine && i == slot) { kr.r[i] = ck; vr.r[i] = cv; }
+        if (mine) { ((uint2*)p.k_pool)[dst] = ck; ((uint2*)p.v_pool)[dst] = cv; }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (mine && i == slot) { kr.r[i] = nk; vr.r[i] = nv; }
+        if (mine) { ((uint4*)p.k_pool)[dst] = nk; ((uint4*)p.v_pool)[dst] = nv; }
+    }
+}
+
 template <bool FP8, bool PAIR>
 __global__ void __launch_bounds__(256, 2)
 paged_decode_mfma_kernel(MfmaParams p) {
@@ -391,6 +448,11 @@ paged_decode_mfma_kernel(MfmaParams p) {
                                                  bb[2], bb[3]);
         }
         const int tile_start = start + tt * TT;
+        // the sequence's newest token lives in this tile (bb still holds its blocks: the last lookup
+        // above was for this wave's final tile)
+        if (p.new_key != nullptr && end == len && tile_start < len && tile_start + TT >= len) {
+            inject_new_row_grid<FP8, PAIR>(kr, vr, p, seq, kvh, lane, tile_start, len, bb);
+        }
         if (tile_start + TT > end)
             process_tile<FP8, false, true, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
                                                  p.hkv, kvh, lane, g4, tile_start, end, cmul);
@@ -489,23 +551,6 @@ struct StreamKParams {
     const bf16_t* new_value;
     int64_t new_token_stride, new_head_stride;     // elements
 };
-
-// 8 floats -> 8 e4m3 codes: clamp(x / scale, +-448), round to nearest even
-__device__ __forceinline__ uint2 quant8_fp8(const uint4& bf, float scale) {
-    const uint32_t w[4] = {bf.x, bf.y, bf.z, bf.w};
-    float f[8];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        f[2 * i] = fminf(fmaxf(__uint_as_float(w[i] << 16) / scale, -448.f), 448.f);
-        f[2 * i + 1] = fminf(fmaxf(__uint_as_float(w[i] & 0xffff0000u) / scale, -448.f), 448.f);
-    }
-    int lo = 0, hi = 0;
-    lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], lo, false);
-    lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
-    hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], hi, false);
-    hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
-    return make_uint2((uint32_t)lo, (uint32_t)hi);
-}
 
 // Fused append: the row's last tile holds the sequence's newest token, whose K/V are not in
 // the pool yet.  The 16 lanes that own that row take it from new_key / new_value instead of
@@ -905,7 +950,7 @@ int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
 
 int launch_decode_mfma(const DecodeArgs& a) {
     MfmaParams p;
-    p.out = a.out; p.query = a.query; p.k_pool = a.k_pool; p.v_pool = a.v_pool;
+    p.out = a.out; p.query = a.query; p.k_pool = (void*)a.k_pool; p.v_pool = (void*)a.v_pool;
     p.block_table = a.block_table; p.block_table_stride = a.block_table_stride;
     p.context_lens = a.context_lens;
     p.hq = a.hq; p.hkv = a.hkv; p.group = a.hq / a.hkv; p.max_blocks = a.max_blocks;
@@ -914,6 +959,8 @@ int launch_decode_mfma(const DecodeArgs& a) {
     p.k_scale = a.k_scale; p.v_scale = a.v_scale;
     p.partition_size = a.partition_size; p.num_parts = a.num_parts;
     p.ws_acc = a.ws.acc; p.ws_ml = a.ws.ml;
+    p.new_key = (const bf16_t*)a.new_key; p.new_value = (const bf16_t*)a.new_value;
+    p.new_token_stride = a.new_token_stride; p.new_head_stride = a.new_head_stride;
     dim3 grid((unsigned)a.hkv, (unsigned)a.num_parts, (unsigned)a.rows);
     const bool fp8 = a.kv_dtype == AICOMP_KV_FP8_E4M3;
     if (a.d == 64) {
