@@ -213,9 +213,7 @@ def test_fused_append_decode_equals_append_then_decode(device, name, batch):
     assert torch.equal(bits(k2), bits(w.k_pool)) and torch.equal(bits(v2), bits(w.v_pool))
     assert torch.equal(out.view(torch.int16 if out.dtype == torch.bfloat16 else torch.int32),
                        ref.view(torch.int16 if ref.dtype == torch.bfloat16 else torch.int32))
-    # explicit partition size: the append runs as its own kernel in front of the grid kernel
-    k3, v3 = k2.clone(), v2.clone()
-    k3.view(torch.uint8).zero_()
+    # explicit partition size: the grid-scheduled kernel (it appends in-kernel too on the matrix-core path)
     ops.paged_decode_attn(out, w.query, k2, v2, w.block_table, w.context_lens, w.scale,
                           k_scale=w.k_scale, v_scale=w.v_scale, new_key=w.new_key, new_value=w.new_value,
                           partition_size=256)
@@ -382,3 +380,31 @@ def test_prepared_decode_equals_the_checked_call(device, name):
         call(torch.empty(5, 3, 7, device=device), w.query)
     with pytest.raises(RuntimeError):
         ops.PreparedDecode(k2, v2, w.block_table.to(torch.int64), w.context_lens, w.query.shape[1], w.query.dtype, w.scale)
+
+
+@pytest.mark.parametrize("d,kv,ps", [(128, None, 64), (128, None, 256), (128, torch.float8_e4m3fn, 128),
+                                     (64, None, 0), (64, None, 128), (64, torch.float8_e4m3fn, 0)])
+def test_fused_append_in_the_grid_kernel_edge_positions(device, d, kv, ps):
+    """The grid-scheduled kernel writes the step's new row itself: new token as the first token, at
+    block, tile (32 / 64 tokens) and partition boundaries, in both halves of a pair row (D = 64).
+    Pools bit-identical to kv_append, output bit-identical to decode after kv_append."""
+    sh = workloads.Shape("t", 12, 8, 2, d, kv_std=0.5, ctx_lo=300, ctx_hi=300,
+                         kv_dtype=kv or torch.bfloat16)
+    w = workloads.make_workload("t", device=device, seed=31, shape=sh)
+    ctx = torch.tensor([1, 2, 16, 17, 32, 33, 64, 65, 128, 129, 257, 300], dtype=torch.int32, device=device)
+    k2, v2 = w.k_pool.clone(), w.v_pool.clone()
+    pos = (ctx - 1).long()
+    slots = w.block_table[torch.arange(12, device=device), pos // 16].long() * 16 + pos % 16
+    ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, slots, w.k_scale, w.v_scale)
+    ref = torch.empty_like(w.query)
+    ops.paged_decode_attn(ref, w.query, w.k_pool, w.v_pool, w.block_table, ctx, w.scale, w.k_scale, w.v_scale,
+                          partition_size=ps)
+    out = torch.full_like(w.query, float("nan"))
+    ops.paged_decode_attn(out, w.query, k2, v2, w.block_table, ctx, w.scale, w.k_scale, w.v_scale,
+                          partition_size=ps, new_key=w.new_key, new_value=w.new_value)
+    torch.cuda.synchronize()
+    assert torch.equal(k2.view(torch.uint8), w.k_pool.view(torch.uint8))
+    assert torch.equal(v2.view(torch.uint8), w.v_pool.view(torch.uint8))
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+    want = oracle_decode(w, ctx=ctx.cpu().numpy())
+    assert_close_attn(to_f64(out), want, BF16_ATOL, BF16_RTOL, f"grid fused append D={d}")
