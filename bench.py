@@ -268,21 +268,31 @@ def prefill_shapes_bench(dev, reps=5):
     import math
     import torch
     from aicomp_amd import ops
-    hq, hkv, d = 32, 8, 128
+    hq, hkv = 32, 8
     out = []
-    for nseq, n, prior in ((1, 8192, 0), (4, 4096, 0), (16, 512, 2048)):
+    for nseq, n, prior, d, fp8 in ((1, 8192, 0, 128, False), (4, 4096, 0, 128, False), (16, 512, 2048, 128, False),
+                                   (16, 512, 2048, 128, True), (16, 512, 2048, 64, False)):
         ctx = prior + n
         nblk = math.ceil(ctx / 16)
         nb = nseq * nblk + 1
         g = torch.Generator().manual_seed(0)
         table = torch.randperm(nb - 1, generator=g)[: nseq * nblk].reshape(nseq, nblk).to(torch.int32).to(dev)
-        k = (torch.randn(nb, hkv, 16, d, device=dev) * 0.5).to(torch.bfloat16)
-        v = (torch.randn(nb, hkv, 16, d, device=dev) * 0.5).to(torch.bfloat16)
+        k = torch.randn(nb, hkv, 16, d, device=dev) * 0.5
+        v = torch.randn(nb, hkv, 16, d, device=dev) * 0.5
+        ks = vs = None
+        if fp8:
+            ks = (k.abs().amax(dim=(0, 2, 3)) / 448).float().contiguous()
+            vs = (v.abs().amax(dim=(0, 2, 3)) / 448).float().contiguous()
+            k = (k / ks[None, :, None, None]).to(torch.float8_e4m3fn)
+            v = (v / vs[None, :, None, None]).to(torch.float8_e4m3fn)
+        else:
+            k, v = k.to(torch.bfloat16), v.to(torch.bfloat16)
         q = torch.randn(nseq * n, hq, d, device=dev).to(torch.bfloat16)
         o = torch.empty_like(q)
         cl = torch.full((nseq,), ctx, dtype=torch.int32, device=dev)
         cu = (torch.arange(nseq + 1, dtype=torch.int32) * n).to(dev)
-        call = lambda: ops.paged_prefill_attn(o, q, k, v, table, cl, cu, 1 / math.sqrt(d), max_q_len=n)
+        call = lambda: ops.paged_prefill_attn(o, q, k, v, table, cl, cu, 1 / math.sqrt(d), max_q_len=n,
+                                              k_scale=ks, v_scale=vs)
         for _ in range(2):
             call()
         e0, e1 = _events(2)
@@ -293,7 +303,8 @@ def prefill_shapes_bench(dev, reps=5):
         torch.cuda.synchronize()
         t = e0.elapsed_time(e1) / reps * 1e-3
         flops = nseq * 4 * hq * d * (n * prior + n * (n + 1) / 2)
-        out.append({"chunks": nseq, "new_tokens": n, "prior": prior, "us": round(t * 1e6, 1),
+        out.append({"chunks": nseq, "new_tokens": n, "prior": prior, "head_dim": d,
+                    "kv_dtype": "float8_e4m3fn" if fp8 else "bfloat16", "us": round(t * 1e6, 1),
                     "TFLOPs": round(flops / t / 1e12, 1),
                     "frac_mfma_peak": round(flops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
         del k, v, q, o
