@@ -42,10 +42,8 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 namespace {
 
-constexpr int D = 128;
 constexpr int BS = 16;
 constexpr int ROWS = 64;               // query rows per workgroup and column group (16 per wave)
-constexpr int KROW = 272;              // LDS row stride in bytes (256 + 16 pad)
 constexpr float NEG_BIG = -1.0e30f;
 
 struct PrefillParams {
@@ -94,36 +92,39 @@ __device__ __forceinline__ float xor32_max(float x) {
     return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 
-template <bool FP8, int KT> struct Stage;
-template <int KT> struct Stage<false, KT> { uint4 k[KT / 16], v[KT / 16]; };
-template <int KT> struct Stage<true, KT> { uint2 k[KT / 16], v[KT / 16]; };
+// register stage of one K and one V tile: NL loads of the workgroup each
+template <bool FP8, int NL> struct Stage;
+template <int NL> struct Stage<false, NL> { uint4 k[NL], v[NL]; };
+template <int NL> struct Stage<true, NL> { uint2 k[NL], v[NL]; };
 
 // R = 16-row column groups per wave (1 or 2).  With R = 2 every K and V operand read from LDS
 // (and every V permute) feeds two MFMAs, and the two groups' softmax chains are independent, so
 // LDS traffic and permute work per flop halve and the scheduler has two chains to interleave.
-// PAIR (head_dim 64): an LDS row is a PAIR of consecutive tokens (token 2r in elements 0..63,
-// token 2r+1 in 64..127, contiguous in the pool), a tile is 64 tokens, and every query row takes
-// two B-operand columns, one per token parity, carrying the query in the matching half of the
-// row and zeros in the other.  The two columns run independent online softmaxes and are merged
-// at the end.  Same instruction stream per byte as head_dim 128, half of it on zeros.
+// DH = head_dim (128 or 64).  An LDS row is one token: 2*DH bytes plus 16 bytes of padding, so that
+// the sixteen rows of an operand read start in different banks (272 B: 4 banks apart; 144 B: 36).
 // KT = rows of an LDS tile (KT/16 blocks): 32 with two register stages for R = 1, 64 with one stage
 // for R = 2, where the per-step work that does not scale with the tile (barrier, block lookups,
 // loop control, the running-max test) is paid half as often.
-template <bool FP8, int R, bool PAIR>
+template <bool FP8, int R, int DH>
 __global__ void __launch_bounds__(256, R == 1 ? 3 : 2)
 paged_prefill_mfma_kernel(PrefillParams p) {
+    constexpr int KROW = 2 * DH + 16;          // LDS row stride in bytes
+    constexpr int NSL = DH / 32;               // 32-element k-slots of a row (QK^T MFMAs per 16 x 16 tile)
+    constexpr int NJ = DH / 16;                // 16-element output tiles (PV MFMAs per 32 tokens)
+    constexpr int CPR = DH / 8;                // 8-element chunks per row
+    constexpr int RPL = 256 / CPR;             // rows one load of the workgroup covers (16 or 32)
     constexpr int KT = R == 1 ? 32 : 64;
     constexpr int NH = KT / 16;                // 16-row groups of a tile
     constexpr int TILE_BYTES = KT * KROW;
-    typedef Stage<FP8, KT> StageT;
+    constexpr int NL = KT / RPL;               // loads per tile and pool
+    typedef Stage<FP8, NL> StageT;
     // Grid: x = head group (fastest: the workgroups of one KV head land on one XCD and share its
     // L2 copy of that head's K/V), y = sequence, z = query tile, longest first (the last tile of a
     // chunk sees the most keys, so it is started first).  Sequence before tile: workgroups that
     // are resident together then come from different chunks, which evens out what a CU is given
     // (measured 102 us against 107 us with the tile index in y on four chunks of 512).
-    constexpr int DQ = PAIR ? 64 : D;          // head_dim of the tensors
-    constexpr int TT = PAIR ? 2 * KT : KT;     // tokens per LDS tile
-    constexpr int CR = PAIR ? 8 : 16;          // query rows per 16-column group
+    constexpr int TT = KT;                     // tokens per LDS tile
+    constexpr int CR = 16;                     // query rows per 16-column group
     constexpr int WROWS = CR * R;              // rows per wave
     const int seq = blockIdx.y;
     const int hgroup = blockIdx.x;
@@ -147,7 +148,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     bool row_valid[R];
 #pragma unroll
     for (int c = 0; c < R; ++c) {
-        const int row = WROWS * w + CR * c + (PAIR ? (r16 >> 1) : r16);
+        const int row = WROWS * w + CR * c + r16;
         qpos[c] = q0 + row / p.gpack;
         head[c] = hgroup * p.gpack + row % p.gpack;
         row_valid[c] = qpos[c] < n;
@@ -162,17 +163,13 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [2][K tile | V tile]
 
     // Q as the B operand: column = this lane's row, k-slots = dims 32s + 8*g4 ..
-    bf16x8_t qf[R][4];
+    bf16x8_t qf[R][NSL];
 #pragma unroll
     for (int c = 0; c < R; ++c) {
-        const bf16_t* qrow = (const bf16_t*)p.query + ((int64_t)(q_begin + min(qpos[c], n - 1)) * p.hq + head[c]) * DQ;
+        const bf16_t* qrow = (const bf16_t*)p.query + ((int64_t)(q_begin + min(qpos[c], n - 1)) * p.hq + head[c]) * DH;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const int e0 = 32 * s + 8 * g4;                     // first element of this k-slot in the LDS row
-            uint4 v = *(const uint4*)(qrow + (PAIR ? (e0 & 63) : e0));
-            if (PAIR && ((e0 >= 64) != ((r16 & 1) != 0))) v = make_uint4(0, 0, 0, 0);
-            qf[c][s] = __builtin_bit_cast(bf16x8_t, v);
-        }
+        for (int s = 0; s < NSL; ++s)                           // k-slot s, k-group g4: elements 32s + 8*g4 ..
+            qf[c][s] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(qrow + 32 * s + 8 * g4));
     }
     // log2(e) * scale * k_scale.  The softmax below tracks the max of the raw scores, which needs
     // a positive multiplier: a negative one (a negative k_scale) moves its sign into Q.
@@ -182,7 +179,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
 #pragma unroll
         for (int c = 0; c < R; ++c)
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
+            for (int s = 0; s < NSL; ++s) {
                 uint4 u = __builtin_bit_cast(uint4, qf[c][s]);
                 u.x ^= 0x80008000u; u.y ^= 0x80008000u; u.z ^= 0x80008000u; u.w ^= 0x80008000u;
                 qf[c][s] = __builtin_bit_cast(bf16x8_t, u);
@@ -191,21 +188,21 @@ paged_prefill_mfma_kernel(PrefillParams p) {
 
     const float lazy_thr = 8.f / cmul;          // +inf for a zero multiplier: every P is 1
     float m[R], lsum[R], bias[R];                // bias = -m * cmul, kept beside m
-    f32x4_t O[R][8];
+    f32x4_t O[R][NJ];
 #pragma unroll
     for (int c = 0; c < R; ++c) {
         m[c] = NEG_BIG; lsum[c] = 0.f; bias[c] = -NEG_BIG * cmul;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) O[c][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < NJ; ++j) O[c][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
 
     typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
     const_i32_ptr table = (const_i32_ptr)(p.block_table + (int64_t)seq * p.block_table_stride);
 
-    // global -> registers: load i of the tile is block (KT/16)*t + i (16 tokens x 16 chunks = 256 lanes);
-    // PAIR: a load covers two 2 KB blocks, waves 0-1 the first, waves 2-3 the second.  The block
-    // ids of a tile are consecutive table entries: one scalar load when all of them exist.
-    constexpr int NB = PAIR ? TT / 16 : KT / 16;               // table entries per tile
+    // global -> registers: one load of the workgroup covers RPL rows of CPR chunks (one block at
+    // D = 128; two blocks at D = 64, waves 0-1 the first, waves 2-3 the second).  The block ids of
+    // a tile are consecutive table entries: one scalar load when all of them exist.
+    constexpr int NB = KT / 16;                                // table entries per tile
     auto fetch = [&](int t, StageT& st) {
         int ids[NB];
         const int first = NB * t;
@@ -220,15 +217,15 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             for (int i = 0; i < NB; ++i) ids[i] = first + i < p.max_blocks ? table[first + i] : 0;
         }
 #pragma unroll
-        for (int i = 0; i < KT / 16; ++i) {
+        for (int i = 0; i < NL; ++i) {
             int b;
-            if constexpr (PAIR) b = (w >> 1) ? ids[2 * i + 1] : ids[2 * i];
+            if constexpr (RPL == 32) b = (w >> 1) ? ids[2 * i + 1] : ids[2 * i];
             else b = ids[i];
             const int blk = max(0, min(b, p.num_blocks - 1));
             // uniform 64-bit base of this head's slice of the block + a constant 32-bit lane offset
             constexpr int ESZ = FP8 ? 1 : 2;
-            const int64_t base = ((int64_t)blk * p.hkv + kvh) * (BS * DQ * ESZ);
-            const int lane_off = (PAIR ? (tid & 127) : tid) * (8 * ESZ);
+            const int64_t base = ((int64_t)blk * p.hkv + kvh) * (BS * DH * ESZ);
+            const int lane_off = (tid & (16 * CPR - 1)) * (8 * ESZ);
             if constexpr (FP8) {
                 st.k[i] = *(const uint2*)((const char*)p.k_pool + base + lane_off);
                 st.v[i] = *(const uint2*)((const char*)p.v_pool + base + lane_off);
@@ -240,23 +237,19 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     };
     // registers -> LDS buffer `buf`.  On the tile that reaches the end of the context, V rows at
     // or beyond it are zeroed (a masked probability of 0 times a non-finite leftover would still
-    // poison the row); PAIR zeroes K there too (the other token of the pair runs its dot products
-    // over the whole row).
+    // poison the row).
     auto stash_rows = [&](int t, int buf, const StageT& st, auto tail_tag) {
         constexpr bool TAIL = decltype(tail_tag)::value;
         unsigned char* kb = lds + buf * 2 * TILE_BYTES;
         unsigned char* vb = kb + TILE_BYTES;
 #pragma unroll
-        for (int i = 0; i < KT / 16; ++i) {
-            const int tok_local = 16 * i + (tid >> 4);           // LDS row
-            const int off = tok_local * KROW + (tid & 15) * 16;
+        for (int i = 0; i < NL; ++i) {
+            const int tok_local = RPL * i + tid / CPR;           // LDS row
+            const int off = tok_local * KROW + (tid % CPR) * 16;
             uint4 kk, vv;
             if constexpr (FP8) { kk = fp8x8_to_bf16x8(st.k[i]); vv = fp8x8_to_bf16x8(st.v[i]); }
             else { kk = st.k[i]; vv = st.v[i]; }
-            if constexpr (TAIL && PAIR) {
-                // chunks 8..15 of a row are the pair's second token
-                if (t * TT + 2 * tok_local + ((tid & 15) >> 3) >= ctx) { kk = make_uint4(0, 0, 0, 0); vv = kk; }
-            } else if constexpr (TAIL) {
+            if constexpr (TAIL) {
                 if (t * KT + tok_local >= ctx) vv = make_uint4(0, 0, 0, 0);
             }
             *(uint4*)(kb + off) = kk;
@@ -294,7 +287,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
 #pragma unroll
             for (int c = 0; c < R; ++c) sa[h][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
+        for (int s = 0; s < NSL; ++s) {
             bf16x8_t a[NH];
 #pragma unroll
             for (int h = 0; h < NH; ++h)
@@ -326,7 +319,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
 #pragma unroll
                 for (int k = 0; k < NS; ++k) {
                     const int r = 16 * (k >> 2) + 4 * (k & 3) + g4;              // LDS row of this score
-                    dead[k] = MASK && sub_start + (PAIR ? 2 * r + (r16 & 1) : r) > qabs[c];
+                    dead[k] = MASK && sub_start + r > qabs[c];
                     if (MASK && dead[k]) sc[k] = NEG_BIG;
                 }
                 float mx_lane = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
@@ -370,7 +363,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         for (int c = 0; c < R; ++c) {
             if (grew[c]) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) O[c][j] *= alpha[c];
+                for (int j = 0; j < NJ; ++j) O[c][j] *= alpha[c];
             }
         }
 
@@ -381,7 +374,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         // by lanes 4e + m/4, e = 0..3, i.e. element 16j + m of four tokens.  Two reads (k-slots
         // 0..3, 4..7) make one operand, which feeds the R column groups.
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < NJ; ++j) {
             typedef short v4i16_t __attribute__((ext_vector_type(4)));
             typedef __attribute__((address_space(3))) v4i16_t* lds_v4i16_ptr;
             typedef short v8i16_t __attribute__((ext_vector_type(8)));
@@ -422,40 +415,18 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         float l = lsum[c];
         l += __shfl_xor(l, 16);
         l += __shfl_xor(l, 32);
-        if constexpr (PAIR) {
-            // merge the row's two parity columns.  Column 2r (even tokens) has its output in
-            // elements 0..63 (j < 4), column 2r+1 in elements 64..127 (j >= 4) of the neighbouring
-            // lane.
-            const float mp = __shfl_xor(m[c], 1), lp = __shfl_xor(l, 1);
-            const float mm = fmaxf(m[c], mp);
-            const float f = __builtin_amdgcn_exp2f((m[c] - mm) * cmul);
-            const float fp = __builtin_amdgcn_exp2f((mp - mm) * cmul);
-            const float lt = l * f + lp * fp;
-            const float inv = (lt > 0.f ? 1.f / lt : 0.f) * (FP8 ? p.v_scale[kvh] : 1.f);
-            const bool writer = row_valid[c] && (r16 & 1) == 0;
-            bf16_t* o = (bf16_t*)p.out + ((int64_t)(q_begin + min(qpos[c], n - 1)) * p.hq + head[c]) * DQ + 4 * g4;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float v[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float other = __shfl_xor(O[c][j + 4][i] * f, 1);     // the odd column's elements 64 + ..
-                    v[i] = (O[c][j][i] * f + other) * inv;
-                }
-                if (writer) *(uint2*)(o + 16 * j) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
-            }
-        } else if (row_valid[c]) {
+        if (row_valid[c]) {
             const float inv = (l > 0.f ? 1.f / l : 0.f) * (FP8 ? p.v_scale[kvh] : 1.f);
-            bf16_t* o = (bf16_t*)p.out + ((int64_t)(q_begin + qpos[c]) * p.hq + head[c]) * D + 4 * g4;
+            bf16_t* o = (bf16_t*)p.out + ((int64_t)(q_begin + qpos[c]) * p.hq + head[c]) * DH + 4 * g4;
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
+            for (int j = 0; j < NJ; ++j)
                 *(uint2*)(o + 16 * j) = make_uint2(pack_bf16(O[c][j][0] * inv, O[c][j][1] * inv),
                                                    pack_bf16(O[c][j][2] * inv, O[c][j][3] * inv));
         }
     }
 }
 
-template <bool FP8, int R, bool PAIR>
+template <bool FP8, int R, int DH>
 static hipError_t launch_prefill_variant(const PrefillParams& p, dim3 grid, size_t lds_bytes, hipStream_t stream) {
     // Two column groups stage 64-row tiles: 70 KB of dynamic LDS, above the 64 KB a kernel may use
     // without asking.  The limit is a per-device function attribute: set once per device.
@@ -465,12 +436,12 @@ static hipError_t launch_prefill_variant(const PrefillParams& p, dim3 grid, size
     if (e != hipSuccess) return e;
     const bool known = dev < 64 && ((done.load(std::memory_order_acquire) >> dev) & 1ull);
     if (!known) {
-        e = hipFuncSetAttribute((const void*)paged_prefill_mfma_kernel<FP8, R, PAIR>,
+        e = hipFuncSetAttribute((const void*)paged_prefill_mfma_kernel<FP8, R, DH>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return e;
         if (dev < 64) done.fetch_or(1ull << dev, std::memory_order_release);
     }
-    hipLaunchKernelGGL((paged_prefill_mfma_kernel<FP8, R, PAIR>), grid, dim3(256), lds_bytes, stream, p);
+    hipLaunchKernelGGL((paged_prefill_mfma_kernel<FP8, R, DH>), grid, dim3(256), lds_bytes, stream, p);
     return hipSuccess;
 }
 
@@ -478,7 +449,7 @@ static hipError_t launch_prefill_variant(const PrefillParams& p, dim3 grid, size
 
 bool prefill_mfma_supported(const DecodeArgs& a, int max_q_len) {
     const int group = a.hkv > 0 ? a.hq / a.hkv : 0;
-    return a.cu_q_lens != nullptr && max_q_len > 0 && (a.d == D || a.d == 64) && a.bs == BS &&
+    return a.cu_q_lens != nullptr && max_q_len > 0 && (a.d == 128 || a.d == 64) && a.bs == BS &&
            a.q_dtype == AICOMP_KV_BF16 &&
            (a.kv_dtype == AICOMP_KV_BF16 || a.kv_dtype == AICOMP_KV_FP8_E4M3) && group >= 1 &&
            a.scale > 0.f && a.num_seqs <= 65535 && ((uintptr_t)a.query % 16 == 0) &&
@@ -498,26 +469,25 @@ int launch_prefill_mfma(const DecodeArgs& a, int max_q_len) {
     p.qk_mul = a.scale * LOG2E;
     p.k_scale = a.k_scale; p.v_scale = a.v_scale;
     // two column groups per wave (128 rows per workgroup) once a chunk has that many rows
-    const bool pair = a.d == 64;                       // head_dim 64: rows of token pairs, 32 query rows per workgroup
-    const int rows1 = pair ? ROWS / 2 : ROWS;
-    const int R = (int64_t)max_q_len * p.gpack >= 2 * rows1 ? 2 : 1;
-    const int pos_per_wg = rows1 * R / p.gpack;
+    const int R = (int64_t)max_q_len * p.gpack >= 2 * ROWS ? 2 : 1;
+    const int pos_per_wg = ROWS * R / p.gpack;
     const int qtiles = (max_q_len + pos_per_wg - 1) / pos_per_wg;
     AICOMP_REQUIRE(qtiles <= 65535, AICOMP_KV_EINVAL, "paged_prefill_attn: grid too large");
     dim3 grid((unsigned)(a.hq / p.gpack), (unsigned)a.num_seqs, (unsigned)qtiles);
-    const size_t lds_bytes = (size_t)4 * (R == 1 ? 32 : 64) * KROW;   // double-buffered K and V tiles
+    // double-buffered K and V tiles of 32 (R = 1) or 64 rows of 2*D + 16 bytes
+    const size_t lds_bytes = (size_t)4 * (R == 1 ? 32 : 64) * (2 * a.d + 16);
     const bool fp8 = a.kv_dtype == AICOMP_KV_FP8_E4M3;
     hipError_t e;
-    if (pair) {
-        if (fp8 && R == 2) e = launch_prefill_variant<true, 2, true>(p, grid, lds_bytes, a.stream);
-        else if (fp8) e = launch_prefill_variant<true, 1, true>(p, grid, lds_bytes, a.stream);
-        else if (R == 2) e = launch_prefill_variant<false, 2, true>(p, grid, lds_bytes, a.stream);
-        else e = launch_prefill_variant<false, 1, true>(p, grid, lds_bytes, a.stream);
+    if (a.d == 64) {
+        if (fp8 && R == 2) e = launch_prefill_variant<true, 2, 64>(p, grid, lds_bytes, a.stream);
+        else if (fp8) e = launch_prefill_variant<true, 1, 64>(p, grid, lds_bytes, a.stream);
+        else if (R == 2) e = launch_prefill_variant<false, 2, 64>(p, grid, lds_bytes, a.stream);
+        else e = launch_prefill_variant<false, 1, 64>(p, grid, lds_bytes, a.stream);
     } else {
-        if (fp8 && R == 2) e = launch_prefill_variant<true, 2, false>(p, grid, lds_bytes, a.stream);
-        else if (fp8) e = launch_prefill_variant<true, 1, false>(p, grid, lds_bytes, a.stream);
-        else if (R == 2) e = launch_prefill_variant<false, 2, false>(p, grid, lds_bytes, a.stream);
-        else e = launch_prefill_variant<false, 1, false>(p, grid, lds_bytes, a.stream);
+        if (fp8 && R == 2) e = launch_prefill_variant<true, 2, 128>(p, grid, lds_bytes, a.stream);
+        else if (fp8) e = launch_prefill_variant<true, 1, 128>(p, grid, lds_bytes, a.stream);
+        else if (R == 2) e = launch_prefill_variant<false, 2, 128>(p, grid, lds_bytes, a.stream);
+        else e = launch_prefill_variant<false, 1, 128>(p, grid, lds_bytes, a.stream);
     }
     AICOMP_REQUIRE(e == hipSuccess, AICOMP_KV_EHIP, "paged_prefill_attn: %s", hipGetErrorString(e));
     AICOMP_HIP_LAUNCH_CHECK();
