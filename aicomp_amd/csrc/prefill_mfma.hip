@@ -106,7 +106,7 @@ template <int NL> struct Stage<true, NL> { uint2 k[NL], v[NL]; };
 // for R = 2, where the per-step work that does not scale with the tile (barrier, block lookups,
 // loop control, the running-max test) is paid half as often.
 template <bool FP8, int R, int DH>
-__global__ void __launch_bounds__(256, R == 1 ? 3 : 2)
+__global__ void __launch_bounds__(256, (R == 1 || DH == 64) ? 3 : 2)
 paged_prefill_mfma_kernel(PrefillParams p) {
     constexpr int KROW = 2 * DH + 16;          // LDS row stride in bytes
     constexpr int NSL = DH / 32;               // 32-element k-slots of a row (QK^T MFMAs per 16 x 16 tile)
