@@ -17,10 +17,10 @@
 //              Groups that do not divide 16 use gpack = 1.  Workgroups of one KV head
 //              are adjacent in the grid (one XCD's L2 serves them); the longest
 //              query tiles of a chunk are launched first.
-// K/V tiles    32 tokens (2 blocks) per step, fetched by the whole workgroup with
-//              coalesced 16-byte loads into registers one tile ahead, written to
-//              a double-buffered LDS tile (row stride 272 B): one barrier per tile,
-//              35 KB of LDS per workgroup.
+// K/V tiles    32 or 64 tokens per step, fetched by the whole workgroup with coalesced
+//              16-byte loads into registers ahead of their use, written to a
+//              double-buffered LDS tile (one padded row per token): one barrier per tile.
+// head_dim     128 or 64, one instantiation each.
 // Per wave     16 or 32 rows (one or two column groups).  S^T = K Q^T with K rows as
 //              the A operand and the wave's query rows as B columns
 //              (v_mfma_f32_16x16x32_bf16); online softmax per column on the raw
