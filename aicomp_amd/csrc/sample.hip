@@ -53,9 +53,11 @@ struct SampleParams {
     int greedy;
 };
 
-// float -> key with the same order (larger float, larger key)
+// float -> key with the same order (larger float, larger key).  -0.0 gets the key of +0.0: the
+// reference compares floats (`logits < kth`), for which the two zeros are one value.
 __device__ __forceinline__ uint32_t order_key(float x) {
-    const uint32_t b = __float_as_uint(x);
+    uint32_t b = __float_as_uint(x);
+    if (b == 0x80000000u) b = 0u;
     return b ^ ((b >> 31) ? 0xffffffffu : 0x80000000u);
 }
 __device__ __forceinline__ float key_value(uint32_t k) {

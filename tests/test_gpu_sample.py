@@ -186,3 +186,14 @@ def test_nucleus_without_top_k_routes(device):
             check_rows(device, x, temperature, 0, top_p)
     check_rows(device, peaked, 0.7, 0, 0.9, dtype=torch.bfloat16)
     check_rows(device, broad, 0.7, 0, 0.9, dtype=torch.bfloat16)
+
+
+def test_signed_zeros_are_one_value(device):
+    """-0.0 and +0.0 compare equal in the reference's float comparisons: when the k-th largest value
+    is a zero, both kinds stay, and they tie in the nucleus order."""
+    rng = np.random.default_rng(12)
+    V = 5000
+    x = (np.round(rng.standard_normal((2, V)) * 1.0) / 2).astype(np.float32)     # many -0.0 and +0.0
+    assert (np.signbit(x) & (x == 0)).sum() > 100 and (~np.signbit(x) & (x == 0)).sum() > 100
+    for temperature, top_k, top_p in [(1.5, 2000, 1.0), (1.5, 2000, 0.9), (1.0, 300, 0.95), (0.7, 0, 0.8)]:
+        check_rows(device, x, temperature, top_k, top_p)
