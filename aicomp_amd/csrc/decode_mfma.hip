@@ -814,32 +814,37 @@ streamk_decode_kernel(StreamKParams p) {
     }
 }
 
-// Merge of the balanced schedule's partials: one wave per (KV head, sequence, head of the
-// group).  The row's partials sit in consecutive slots first+row .. last+row (first / last
-// wave recorded by the main kernel); their weights 2^(m_i - M) are computed once (one lane
-// per partial) and parked in LDS, then each lane accumulates two output dims with
-// independent loads.  One wave per head: reductions are shuffles, no barrier.
-constexpr int RED_WGT = 256;       // weights parked in LDS per head; rows with more partials recompute the rest
+// Merge of the balanced schedule's partials: one workgroup per (KV head, sequence), S waves per
+// head of the group.  The row's partials sit in consecutive slots first+row .. last+row (first /
+// last wave recorded by the main kernel); their weights 2^(m_i - M) are computed once (one lane
+// per partial) and parked in LDS, then each lane accumulates two output dims with independent
+// loads.  With S = 1 (few partials per row, the usual batch) reductions are shuffles and there is
+// no barrier; with S > 1 (a handful of very long rows, hundreds of partials each) the waves of a
+// head take alternate groups of eight partials and add up through LDS.
+constexpr int RED_WGT = 256;       // weights parked in LDS per wave; rows with more partials recompute the rest
 __global__ void __launch_bounds__(1024)
 streamk_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws_acc,
                       const float* __restrict__ ws_ml, const int* __restrict__ ws_rows,
                       const int32_t* __restrict__ context_lens, int hq, int hkv, int group,
                       const float* __restrict__ v_scale) {
-    // one workgroup per (KV head, sequence), one wave per head of the group
-    const int kvh = blockIdx.x, seq = blockIdx.y, h = threadIdx.x >> 6;
+    const int kvh = blockIdx.x, seq = blockIdx.y, wv = threadIdx.x >> 6;
+    const int S = (int)(blockDim.x >> 6) / group;          // waves per head
+    const int h = wv / S, sub = wv % S;
     const int lane = threadIdx.x & 63;
     __shared__ float wgt_all[16][RED_WGT];
-    float* wgt = wgt_all[h];
+    __shared__ float part[16][D];
+    float* wgt = wgt_all[wv];
     const int64_t row = (int64_t)seq * hkv + kvh;
     bf16_t* o = out + ((int64_t)seq * hq + kvh * group + h) * D;
-    if (context_lens[seq] <= 0) {            // no tiles, no partials: the output row is zero
-        o[lane].bits = 0; o[lane + 64].bits = 0;
+    if (context_lens[seq] <= 0) {            // no tiles, no partials: the output row is zero (whole workgroup)
+        if (sub == 0) { o[lane].bits = 0; o[lane + 64].bits = 0; }
         return;
     }
     const int first = ws_rows[2 * row], last = ws_rows[2 * row + 1];
     const int np = last - first + 1;
     const float* ml = ws_ml + ((first + row) * group + h) * 2;          // partial i at ml[i * group * 2]
     const float* acc = ws_acc + ((first + row) * group + h) * D + lane; // partial i at acc[i * group * D]
+    // every wave of a head computes the row's max, denominator and weights for itself (np / 64 loads per lane)
     float mx = NEG_BIG;
     for (int i = lane; i < np; i += 64) mx = fmaxf(mx, ml[(int64_t)i * group * 2]);
 #pragma unroll
@@ -854,10 +859,9 @@ streamk_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws_acc
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) den += __shfl_xor(den, off);
     const int64_t stride = (int64_t)group * D;
-    // eight partials (sixteen loads) in flight per step: a long row has tens of partials and
-    // the loop is pure load latency
+    // eight partials (sixteen loads) in flight per step: the loop is pure load latency
     float n0 = 0.f, n1 = 0.f;
-    for (int i0 = 0; i0 < np; i0 += 8) {
+    for (int i0 = 8 * sub; i0 < np; i0 += 8 * S) {
         float a[8], b[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
@@ -872,6 +876,12 @@ streamk_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws_acc
             n0 = fmaf(f, a[u], n0);
             n1 = fmaf(f, b[u], n1);
         }
+    }
+    if (S > 1) {                             // workgroup-uniform
+        part[wv][lane] = n0; part[wv][lane + 64] = n1;
+        __syncthreads();
+        if (sub != 0) return;
+        for (int k = 1; k < S; ++k) { n0 += part[wv + k][lane]; n1 += part[wv + k][lane + 64]; }
     }
     const float inv = den > 0.f ? (v_scale ? v_scale[kvh] : 1.f) / den : 0.f;
     o[lane].bits = f32_to_bf16(n0 * inv);
@@ -941,7 +951,10 @@ int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
     else
         hipLaunchKernelGGL(streamk_decode_kernel<false>, dim3(wgs), dim3(256), 0, a.stream, p);
     AICOMP_HIP_LAUNCH_CHECK();
-    hipLaunchKernelGGL(streamk_reduce_kernel, dim3(a.hkv, (unsigned)a.rows), dim3(64 * group), 0, a.stream,
+    // waves per head in the merge: one, unless rows are few and long (many partials per row)
+    const int64_t per_row = (int64_t)p.num_waves / (a.rows * a.hkv) + 2;
+    const int sub = per_row > 8 ? 16 / group : 1;
+    hipLaunchKernelGGL(streamk_reduce_kernel, dim3(a.hkv, (unsigned)a.rows), dim3(64 * group * sub), 0, a.stream,
                        (bf16_t*)a.out, p.ws_acc, p.ws_ml, p.ws_rows, a.context_lens, a.hq, a.hkv, group,
                        a.v_scale);
     AICOMP_HIP_LAUNCH_CHECK();
