@@ -103,3 +103,51 @@ def test_random_operator_sessions(device, seed):
             assert bool(ok.all()), f"{what}: n {n} at {pos}: max abs err {err.max().item():.3e}"
             pos += n
         new.disable()
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_sampler_rows(device, seed):
+    """Random vocabulary sizes, row shapes (Gaussian, peaked, nearly flat, heavily tied incl. signed
+    zeros, masked with -inf), temperatures, top-k / top-p and logit types against the oracle.  A
+    probability below the kernel's fixed-point resolution (2^-40 of the row maximum) may be zero."""
+    from oracle import sample_oracle as S
+    rnd = random.Random(300 + seed)
+    for trial in range(40):
+        V = rnd.choice([1, 2, 17, 64, 500, 1024, 1025, 5000, 33000])
+        B = rnd.choice([1, 3])
+        rng = np.random.default_rng(1000 * seed + trial)
+        kind = rnd.choice(["gauss", "peaked", "flat", "ties", "masked"])
+        x = (rng.standard_normal((B, V)) * rnd.choice([0.5, 2.0, 4.0])).astype(np.float32)
+        if kind == "peaked" and V > 40:
+            for b in range(B):
+                x[b, rng.choice(V, min(30, V // 2), replace=False)] += 12
+        elif kind == "flat":
+            x = (rng.standard_normal((B, V)) * 0.01).astype(np.float32)
+        elif kind == "ties":
+            x = (np.round(x * 2) / 2).astype(np.float32)
+        elif kind == "masked" and V > 4:
+            for b in range(B):
+                x[b, rng.choice(V, V * 3 // 4, replace=False)] = -np.inf
+        T = rnd.choice([1.0, 0.7, 1.5, 0.3, 5.0])
+        top_k = rnd.choice([0, 0, 1, 5, 50, 1000, 2000, V, V + 5])
+        top_p = rnd.choice([1.0, 0.9, 0.5, 0.99, 0.0, 0.3])
+        dtype = rnd.choice([torch.float32, torch.float32, torch.bfloat16])
+        what = f"seed {seed} trial {trial}: V {V}, {kind}, T {T}, top_k {top_k}, top_p {top_p}, {dtype}"
+        u = torch.rand(B, generator=torch.Generator().manual_seed(trial))
+        xt = torch.from_numpy(x).to(dtype)
+        name = "bf16" if dtype == torch.bfloat16 else "f32"
+        vals = xt.float().numpy()
+        tok, probs = ops.sample_tokens(xt.to(device), T, top_k, top_p, True, u.to(device), return_probs=True)
+        tok, probs = tok.cpu().numpy(), probs.cpu().numpy().astype(np.float64)
+        for b in range(B):
+            want = S.filtered_probs(vals[b], T, top_k, top_p, name)
+            margin = S.nucleus_margin(vals[b], T, top_k, top_p, name) if top_p < 1 else np.full(V, np.inf)
+            sure = (margin > 2e-5) & ((want > 1e-11) | (want == 0))
+            assert np.array_equal((probs[b] > 0)[sure], (want > 0)[sure]), f"{what}, row {b}: kept set differs"
+            assert abs(probs[b].sum() - 1) < 1e-5, what
+            if np.array_equal(probs[b] > 0, want > 0):
+                assert np.allclose(probs[b], want, rtol=3e-5, atol=1e-9), f"{what}, row {b}: probabilities differ"
+            cdf, t = np.cumsum(probs[b]), int(tok[b])
+            assert probs[b, t] > 0, f"{what}, row {b}: token {t} has no mass"
+            lo = cdf[t - 1] if t else 0.0
+            assert lo - 1e-6 <= float(u[b]) <= cdf[t] + 1e-6, f"{what}, row {b}: draw outside its CDF step"
