@@ -49,6 +49,22 @@ def build(verbose: bool = True, jobs: int = 7) -> str:
     return LIB
 
 
+def build_host_example(verbose: bool = True) -> str:
+    """Compile tests/cabi_host.cpp, a C++ program that links the library directly (no Python, no
+    torch): the boundary as a C or C++ host sees it."""
+    root = os.path.dirname(HERE)
+    src, exe = os.path.join(root, "tests", "cabi_host.cpp"), os.path.join(root, "tests", "cabi_host")
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-I" + os.path.join(root, "include"), src,
+           "-L" + HERE, "-laicomp_kv", "-Wl,-rpath,$ORIGIN/../aicomp_amd", "-o", exe]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")
+    if verbose:
+        print(f"built {exe}")
+    return exe
+
+
 if __name__ == "__main__":
     build()
+    build_host_example()
     sys.exit(0)
