@@ -17,15 +17,19 @@
 //              Groups that do not divide 16 use gpack = 1.  Workgroups of one KV head
 //              are adjacent in the grid (one XCD's L2 serves them); the longest
 //              query tiles of a chunk are launched first.
-// K/V tiles    32 or 64 tokens per step, fetched by the whole workgroup with coalesced
-//              16-byte loads into registers ahead of their use, written to a
-//              double-buffered LDS tile (one padded row per token): one barrier per tile.
+// K/V tiles    32 or 64 tokens per step, double-buffered in LDS, one barrier per tile.  bf16
+//              pools with D = 128 and two column groups: loaded straight into LDS
+//              (global_load_lds_dwordx4, 1 KB = four token rows per wave instruction) one tile
+//              ahead, rows unpadded with their 16-byte chunks XOR-swizzled by the row index.
+//              Otherwise: coalesced 16-byte loads into registers ahead of their use, written
+//              to LDS (one padded row per token; fp8 is widened to bf16 on the way).
 // head_dim     128 or 64, one instantiation each.
 // Per wave     16 or 32 rows (one or two column groups).  S^T = K Q^T with K rows as
 //              the A operand and the wave's query rows as B columns
 //              (v_mfma_f32_16x16x32_bf16); online softmax per column on the raw
-//              scores with a lazily moved max, lane-local except the row max (two
-//              lane swaps); O^T += V^T P^T with the V^T operand read out of the row-major
+//              scores with a lazily moved max: the exponentials are taken against the current
+//              max and their sum tells whether it has to move (then, rarely, the row max is
+//              found with two lane swaps and the exponentials are redone); O^T += V^T P^T with the V^T operand read out of the row-major
 //              V tile by gfx950's transposing LDS read (ds_read_b64_tr_b16), in the token
 //              order the QK product was laid out in, so P never leaves its lane.  With two
 //              column groups every LDS operand read feeds two MFMAs.
@@ -105,10 +109,18 @@ template <int NL> struct Stage<true, NL> { uint2 k[NL], v[NL]; };
 // KT = rows of an LDS tile (KT/16 blocks): 32 with two register stages for R = 1, 64 with one stage
 // for R = 2, where the per-step work that does not scale with the tile (barrier, block lookups,
 // loop control, the running-max test) is paid half as often.
-template <bool FP8, int R, int DH>
+// DMA = tiles go from the pool straight into LDS (bf16, R = 2, D = 128): no staging registers, no
+// LDS writes by the waves.  The two buffers are separate __shared__ arrays and every read address
+// is one offset from its array, which is what lets the compiler see that a read of one buffer
+// need not wait for the loads in flight into the other; the only wait is at the barrier that
+// opens a step, for the loads issued one step earlier.
+#define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+template <bool FP8, int R, int DH, bool DMA>
 __global__ void __launch_bounds__(256, (R == 1 || DH == 64) ? 3 : 2)
 paged_prefill_mfma_kernel(PrefillParams p) {
-    constexpr int KROW = 2 * DH + 16;          // LDS row stride in bytes
+    static_assert(!DMA || (!FP8 && R == 2 && DH == 128), "direct-to-LDS tiles: bf16, two column groups, D = 128");
+    constexpr int KROW = DMA ? 2 * DH : 2 * DH + 16;          // LDS row stride in bytes
     constexpr int NSL = DH / 32;               // 32-element k-slots of a row (QK^T MFMAs per 16 x 16 tile)
     constexpr int NJ = DH / 16;                // 16-element output tiles (PV MFMAs per 32 tokens)
     constexpr int CPR = DH / 8;                // 8-element chunks per row
@@ -161,6 +173,12 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     const int ntiles = (kv_end + TT - 1) / TT;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [2][K tile | V tile]
+    // Direct-to-LDS tiles: four separate arrays, so that the compiler can tell a read of one
+    // buffer from the loads in flight into the other.
+    __shared__ __attribute__((aligned(16))) unsigned char dma_k0[DMA ? TILE_BYTES : 16];
+    __shared__ __attribute__((aligned(16))) unsigned char dma_v0[DMA ? TILE_BYTES : 16];
+    __shared__ __attribute__((aligned(16))) unsigned char dma_k1[DMA ? TILE_BYTES : 16];
+    __shared__ __attribute__((aligned(16))) unsigned char dma_v1[DMA ? TILE_BYTES : 16];
 
     // Q as the B operand: column = this lane's row, k-slots = dims 32s + 8*g4 ..
     bf16x8_t qf[R][NSL];
@@ -186,7 +204,6 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             }
     }
 
-    const float lazy_thr = 8.f / cmul;          // +inf for a zero multiplier: every P is 1
     float m[R], lsum[R], bias[R];                // bias = -m * cmul, kept beside m
     f32x4_t O[R][NJ];
 #pragma unroll
@@ -261,7 +278,9 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         else stash_rows(t, buf, st, std::false_type{});
     };
 
-    const int rd_k = (4 * (r16 & 3) + (r16 >> 2)) * KROW + g4 * 16;   // permuted K row, chunk g4
+    const int prow = 4 * (r16 & 3) + (r16 >> 2);                       // permuted K row
+    const int rd_k = prow * KROW + g4 * 16;                            // chunk g4
+    const int vrow = 4 * (r16 >> 2) + g4;
     // transposing V read: lane k of a 16-lane group addresses token row 4*(k/4) + g4, elements 4*(k%4) ..
     const int rd_v = (4 * (r16 >> 2) + g4) * KROW + (r16 & 3) * 8;
 
@@ -269,14 +288,67 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     // stages of 32 rows: tile t+2; one stage of 64 rows: tile t+1), so a tile's loads have the
     // time of 64 rows of arithmetic to land.
     constexpr int AHEAD = KT == 32 ? 2 : 1;
-    auto step = [&](int t, StageT& st) {
+    // Direct-to-LDS fetch of tile t: each wave instruction lands 1 KB = four 256-byte rows, lane l
+    // at row 4w + l/16 of block i, chunk slot l%16; the slot holds chunk (l%16) ^ row (the XOR
+    // swizzle that keeps the operand reads free of bank conflicts without padding), so the lane
+    // reads that chunk from the pool.
+    const int dma_row = 4 * w + g4;
+    const uint32_t dma_blk_stride = (uint32_t)p.hkv * (BS * DH * 2);              // bytes per block, < 2^32
+    const char* dma_kp = (const char*)p.k_pool + (int64_t)kvh * (BS * DH * 2);   // this KV head's slice of block 0
+    const char* dma_vp = (const char*)p.v_pool + (int64_t)kvh * (BS * DH * 2);
+    auto fetch_dma = [&](int t, unsigned char* kb, unsigned char* vb) {
+        const int first = NB * t;
+        const bool tail = (t + 1) * KT > ctx || first + NB > p.max_blocks;     // workgroup-uniform
+        if (!tail) {
+            typedef int idvec_t __attribute__((ext_vector_type(NB), aligned(4)));
+            typedef const __attribute__((address_space(4))) idvec_t* const_idvec_ptr;
+            const idvec_t v = *(const_idvec_ptr)(table + first);
+            uint32_t lane_off = dma_row * (2 * DH) + ((r16 ^ dma_row) << 4);
+            // opaque per step: keeps the address a uniform 64-bit base plus this 32-bit lane offset
+            // (the load's scalar-base form) instead of a hoisted per-lane 64-bit pointer
+            asm volatile("" : "+v"(lane_off));
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                const uint32_t blk = min((uint32_t)v[i], (uint32_t)(p.num_blocks - 1));
+                const uint64_t base = (uint64_t)blk * dma_blk_stride;
+                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(dma_kp + base + lane_off),
+                                                 LDS_PTR(kb + (16 * i + 4 * w) * KROW), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(dma_vp + base + lane_off),
+                                                 LDS_PTR(vb + (16 * i + 4 * w) * KROW), 16, 0, 0);
+            }
+        } else {
+            // rows at or beyond the context take the last valid row instead (finite data for
+            // the masked probabilities of 0 to multiply)
+            const int last = ctx - 1, last_blk = last >> 4;
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                const int bi = min(first + i, last_blk);
+                const int blk = max(0, min(table[bi], p.num_blocks - 1));
+                const int64_t base = ((int64_t)blk * p.hkv + kvh) * (BS * DH * 2);
+                const int tok = min(16 * (first + i) + dma_row, last);
+                const uint32_t lane_off = (tok - 16 * bi) * (2 * DH) + ((r16 ^ dma_row) << 4);
+                __builtin_amdgcn_global_load_lds(GLOBAL_PTR((const char*)p.k_pool + base + lane_off),
+                                                 LDS_PTR(kb + (16 * i + 4 * w) * KROW), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds(GLOBAL_PTR((const char*)p.v_pool + base + lane_off),
+                                                 LDS_PTR(vb + (16 * i + 4 * w) * KROW), 16, 0, 0);
+            }
+        }
+    };
+    auto step = [&](int t, StageT& st, unsigned char* kb_, unsigned char* vb_, unsigned char* kn, unsigned char* vn) {
         const int buf = t & 1;
-        stash(t, buf, st);
-        fetch(min(t + AHEAD, ntiles - 1), st);  // unconditional: a static count of loads in flight
-        __syncthreads();          // tile t visible; everyone is done with the buffer tile t+1 will use
-
-        const unsigned char* kb = lds + buf * 2 * TILE_BYTES;
-        const unsigned char* vb = kb + TILE_BYTES;
+        const unsigned char* kb;
+        const unsigned char* vb;
+        if constexpr (DMA) {
+            __syncthreads();      // tile t has landed (own loads waited for, then everyone's); tile t-1 is no longer read
+            if (t + 1 < ntiles) fetch_dma(t + 1, kn, vn);
+            kb = kb_; vb = vb_;
+        } else {
+            stash(t, buf, st);
+            fetch(min(t + AHEAD, ntiles - 1), st);  // unconditional: a static count of loads in flight
+            __syncthreads();          // tile t visible; everyone is done with the buffer tile t+1 will use
+            kb = lds + buf * 2 * TILE_BYTES;
+            vb = kb + TILE_BYTES;
+        }
         const int sub_start = t * TT;
         if (sub_start >= wave_kv_end) return;                          // wave-uniform: above the diagonal
 
@@ -291,7 +363,10 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             bf16x8_t a[NH];
 #pragma unroll
             for (int h = 0; h < NH; ++h)
-                a[h] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kb + 16 * h * KROW + rd_k + s * 64));
+                if constexpr (DMA)   // chunk 4s + g4 of row 16h + prow sits at chunk slot (4s + g4) ^ prow
+                    a[h] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kb + 16 * h * KROW + prow * KROW + (((4 * s + g4) ^ prow) << 4)));
+                else
+                    a[h] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kb + 16 * h * KROW + rd_k + s * 64));
 #pragma unroll
             for (int h = 0; h < NH; ++h)
 #pragma unroll
@@ -299,10 +374,10 @@ paged_prefill_mfma_kernel(PrefillParams p) {
                     sa[h][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[h], qf[c][s], sa[h][c], 0, 0, 0);
         }
         // Online softmax on the raw scores: the score multiplier is folded into the exponent's
-        // fused multiply-add and the running max stays in raw units.  The max is only moved when a
-        // row's new maximum exceeds it by more than 2^8 after scaling: until then P is at most
-        // 256, exact enough in bf16 and f32, and the accumulators need no rescale.  Only tiles that
-        // cross the diagonal pay for the mask.
+        // fused multiply-add and the running max stays in raw units.  The max is moved lazily:
+        // the exponentials are first taken against the current max, and as long as a lane's sum of
+        // them stays <= 2^8 every P is at most 256, exact enough in bf16 and f32, and neither the
+        // max nor the accumulators are touched.  Only tiles that cross the diagonal pay for the mask.
         const bool need_mask = sub_start + TT - 1 > wave_kv_min;       // wave-uniform
         bf16x8_t pf[R][NH / 2];
         float alpha[R];
@@ -322,38 +397,52 @@ paged_prefill_mfma_kernel(PrefillParams p) {
                     dead[k] = MASK && sub_start + r > qabs[c];
                     if (MASK && dead[k]) sc[k] = NEG_BIG;
                 }
-                float mx_lane = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
-                                      fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-                if constexpr (NS == 16)
-                    mx_lane = fmaxf(mx_lane, fmaxf(fmaxf(fmaxf(sc[8], sc[9]), fmaxf(sc[10], sc[11])),
-                                                   fmaxf(fmaxf(sc[12], sc[13]), fmaxf(sc[14], sc[15]))));
+                // Exponentials against the current reference max, rounded to bf16 in pairs; the sum
+                // of the rounded pairs (v_dot2c_f32_bf16 against ones: one instruction per two
+                // probabilities, and the sum of exactly what the PV product multiplies) doubles as
+                // the test that none of them outgrew the max.  The first tile always fails it (the
+                // initial max is -1e30); a NaN sum is carried through on either path.
+                uint32_t pk[NS / 2];
+                float psum = 0.f;
+                auto exps = [&]() {
+                    psum = 0.f;
+#pragma unroll
+                    for (int k = 0; k < NS; k += 2) {
+                        float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[k], cmul, bias[c]));
+                        float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[k + 1], cmul, bias[c]));
+                        if (MASK && dead[k]) p0 = 0.f;
+                        if (MASK && dead[k + 1]) p1 = 0.f;
+                        const bf16x2_t pp = {(__bf16)p0, (__bf16)p1};
+                        const bf16x2_t one = {(__bf16)1.0f, (__bf16)1.0f};
+                        psum = __builtin_amdgcn_fdot2_f32_bf16(pp, one, psum, false);
+                        pk[k >> 1] = __builtin_bit_cast(uint32_t, pp);
+                    }
+                };
+                exps();
                 // A row's scores sit in four lanes (l, l^16, l^32, l^48), which must share one
-                // reference max.  It can only have to move if some lane's own maximum outgrows it,
-                // so the exchange, the rescale factor and the accumulator rescale (below) all sit
-                // behind one wave-uniform test that is false on almost every tile after the first.
-                grew[c] = __any(mx_lane - m[c] > lazy_thr);
+                // reference max, so the whole wave takes the slow path together: row max over the
+                // lanes, rescale factor, exponentials again (the accumulator rescale is below).
+                grew[c] = __any(!(psum <= 256.f));
                 if (grew[c]) {
+                    float mx_lane = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
+                                          fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+                    if constexpr (NS == 16)
+                        mx_lane = fmaxf(mx_lane, fmaxf(fmaxf(fmaxf(sc[8], sc[9]), fmaxf(sc[10], sc[11])),
+                                                       fmaxf(fmaxf(sc[12], sc[13]), fmaxf(sc[14], sc[15]))));
                     float mx = xor16_max(mx_lane);
                     mx = xor32_max(mx);
-                    const bool up = mx - m[c] > lazy_thr;
+                    const bool up = mx > m[c];
                     alpha[c] = up ? __builtin_amdgcn_exp2f((m[c] - mx) * cmul) : 1.f;
                     m[c] = up ? mx : m[c];
                     bias[c] = -m[c] * cmul;
                     lsum[c] *= alpha[c];
-                }
-                float pr[NS], psum;
-#pragma unroll
-                for (int k = 0; k < NS; ++k) {
-                    pr[k] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[k], cmul, bias[c]));
-                    if (MASK && dead[k]) pr[k] = 0.f;
-                    psum = k ? psum + pr[k] : pr[k];
+                    exps();
                 }
                 lsum[c] += psum;
 #pragma unroll
                 for (int hp = 0; hp < NH / 2; ++hp) {
                     uint4 pw;
-                    pw.x = pack_bf16(pr[8 * hp + 0], pr[8 * hp + 1]); pw.y = pack_bf16(pr[8 * hp + 2], pr[8 * hp + 3]);
-                    pw.z = pack_bf16(pr[8 * hp + 4], pr[8 * hp + 5]); pw.w = pack_bf16(pr[8 * hp + 6], pr[8 * hp + 7]);
+                    pw.x = pk[4 * hp + 0]; pw.y = pk[4 * hp + 1]; pw.z = pk[4 * hp + 2]; pw.w = pk[4 * hp + 3];
                     pf[c][hp] = __builtin_bit_cast(bf16x8_t, pw);
                 }
             }
@@ -380,9 +469,10 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             typedef short v8i16_t __attribute__((ext_vector_type(8)));
 #pragma unroll
             for (int hp = 0; hp < NH / 2; ++hp) {
-                const unsigned char* vt = vb + 32 * hp * KROW + rd_v + j * 32;
-                const v4i16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)vt);
-                const v4i16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(vt + 16 * KROW));
+                const int voff = DMA ? 32 * hp * KROW + vrow * KROW + (((2 * j + ((r16 >> 1) & 1)) ^ vrow) << 4) + (r16 & 1) * 8
+                                     : 32 * hp * KROW + rd_v + j * 32;
+                const v4i16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(vb + voff));
+                const v4i16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(vb + (voff + 16 * KROW)));
                 const v8i16_t av = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 const bf16x8_t a = __builtin_bit_cast(bf16x8_t, av);
 #pragma unroll
@@ -395,18 +485,25 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     // a fixed number of loads in flight the wait before a stage is written to LDS covers that
     // stage's loads only, not the younger ones of the other stage.  With two stages the loop
     // always runs both; a step past the last tile stages it again and skips the arithmetic.
-    if constexpr (KT == 32) {
+    if constexpr (DMA) {
+        StageT st;
+        fetch_dma(0, dma_k0, dma_v0);
+        for (int t = 0; t < ntiles; t += 2) {
+            step(t, st, dma_k0, dma_v0, dma_k1, dma_v1);
+            if (t + 1 < ntiles) step(t + 1, st, dma_k1, dma_v1, dma_k0, dma_v0);
+        }
+    } else if constexpr (KT == 32) {
         StageT st_a, st_b;
         fetch(0, st_a);
         fetch(min(1, ntiles - 1), st_b);
         for (int t = 0; t < ntiles; t += 2) {
-            step(t, st_a);
-            step(t + 1, st_b);
+            step(t, st_a, nullptr, nullptr, nullptr, nullptr);
+            step(t + 1, st_b, nullptr, nullptr, nullptr, nullptr);
         }
     } else {
         StageT st;
         fetch(0, st);
-        for (int t = 0; t < ntiles; ++t) step(t, st);
+        for (int t = 0; t < ntiles; ++t) step(t, st, nullptr, nullptr, nullptr, nullptr);
     }
 
     // lane (column r16 of column group c, g4) holds O^T[element 16*j + 4*g4 + i][column] in O[c][j][i]
@@ -426,7 +523,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     }
 }
 
-template <bool FP8, int R, int DH>
+template <bool FP8, int R, int DH, bool DMA = false>
 static hipError_t launch_prefill_variant(const PrefillParams& p, dim3 grid, size_t lds_bytes, hipStream_t stream) {
     // Two column groups stage 64-row tiles: 70 KB of dynamic LDS, above the 64 KB a kernel may use
     // without asking.  The limit is a per-device function attribute: set once per device.
@@ -436,12 +533,12 @@ static hipError_t launch_prefill_variant(const PrefillParams& p, dim3 grid, size
     if (e != hipSuccess) return e;
     const bool known = dev < 64 && ((done.load(std::memory_order_acquire) >> dev) & 1ull);
     if (!known) {
-        e = hipFuncSetAttribute((const void*)paged_prefill_mfma_kernel<FP8, R, DH>,
+        e = hipFuncSetAttribute((const void*)paged_prefill_mfma_kernel<FP8, R, DH, DMA>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return e;
         if (dev < 64) done.fetch_or(1ull << dev, std::memory_order_release);
     }
-    hipLaunchKernelGGL((paged_prefill_mfma_kernel<FP8, R, DH>), grid, dim3(256), lds_bytes, stream, p);
+    hipLaunchKernelGGL((paged_prefill_mfma_kernel<FP8, R, DH, DMA>), grid, dim3(256), lds_bytes, stream, p);
     return hipSuccess;
 }
 
@@ -486,7 +583,7 @@ int launch_prefill_mfma(const DecodeArgs& a, int max_q_len) {
     } else {
         if (fp8 && R == 2) e = launch_prefill_variant<true, 2, 128>(p, grid, lds_bytes, a.stream);
         else if (fp8) e = launch_prefill_variant<true, 1, 128>(p, grid, lds_bytes, a.stream);
-        else if (R == 2) e = launch_prefill_variant<false, 2, 128>(p, grid, lds_bytes, a.stream);
+        else if (R == 2) e = launch_prefill_variant<false, 2, 128, true>(p, grid, 0, a.stream);   // static LDS
         else e = launch_prefill_variant<false, 1, 128>(p, grid, lds_bytes, a.stream);
     }
     AICOMP_REQUIRE(e == hipSuccess, AICOMP_KV_EHIP, "paged_prefill_attn: %s", hipGetErrorString(e));

@@ -100,7 +100,8 @@ def test_adapter_chunked_prefill_is_causal(device):
     chunk = a(q1, ex(k1), ex(v1))
     for i in range(9):
         step = b(q1[:, :, i:i + 1], ex(k1[:, :, i:i + 1]), ex(v1[:, :, i:i + 1]))
-        assert (step[:, :, 0].float() - chunk[:, :, i].float()).abs().max() <= 4e-3
+        # two kernels, two summation orders: at most one bf16 ulp of an output in [1, 2)
+        assert (step[:, :, 0].float() - chunk[:, :, i].float()).abs().max() <= 2.0 ** -7
     assert a.cache_pos == b.cache_pos == 29
 
 
