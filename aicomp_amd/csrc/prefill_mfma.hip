@@ -288,49 +288,51 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     // stages of 32 rows: tile t+2; one stage of 64 rows: tile t+1), so a tile's loads have the
     // time of 64 rows of arithmetic to land.
     constexpr int AHEAD = KT == 32 ? 2 : 1;
-    // Direct-to-LDS fetch of tile t: each wave instruction lands 1 KB = four 256-byte rows, lane l
-    // at row 4w + l/16 of block i, chunk slot l%16; the slot holds chunk (l%16) ^ row (the XOR
-    // swizzle that keeps the operand reads free of bank conflicts without padding), so the lane
-    // reads that chunk from the pool.
-    const int dma_row = 4 * w + g4;
+    // Direct-to-LDS fetch of tile t: wave w brings in block w of the tile (16 token rows of 256
+    // bytes) with four instructions of 1 KB each; lane l of instruction q lands at row 4q + l/16,
+    // chunk slot l%16, and the slot holds chunk (l%16) ^ row (the XOR swizzle that keeps the
+    // operand reads free of bank conflicts without padding), so the lane reads that chunk from the
+    // pool.  One block per wave: one table entry, one base address and one LDS base per pool; the
+    // instruction's immediate offset moves the pool and the LDS address together by 1 KB per q.
+    static_assert(!DMA || NB == 4, "one block of the tile per wave");
     const uint32_t dma_blk_stride = (uint32_t)p.hkv * (BS * DH * 2);              // bytes per block, < 2^32
     const char* dma_kp = (const char*)p.k_pool + (int64_t)kvh * (BS * DH * 2);   // this KV head's slice of block 0
     const char* dma_vp = (const char*)p.v_pool + (int64_t)kvh * (BS * DH * 2);
+    uint32_t dma_off[4];                       // pool offset of this lane's chunk, less the immediate
+#pragma unroll
+    for (int q = 0; q < 4; ++q) dma_off[q] = g4 * (2 * DH) + ((r16 ^ g4 ^ (4 * q)) << 4);
     auto fetch_dma = [&](int t, unsigned char* kb, unsigned char* vb) {
         const int first = NB * t;
         const bool tail = (t + 1) * KT > ctx || first + NB > p.max_blocks;     // workgroup-uniform
         if (!tail) {
-            typedef int idvec_t __attribute__((ext_vector_type(NB), aligned(4)));
-            typedef const __attribute__((address_space(4))) idvec_t* const_idvec_ptr;
-            const idvec_t v = *(const_idvec_ptr)(table + first);
-            uint32_t lane_off = dma_row * (2 * DH) + ((r16 ^ dma_row) << 4);
-            // opaque per step: keeps the address a uniform 64-bit base plus this 32-bit lane offset
-            // (the load's scalar-base form) instead of a hoisted per-lane 64-bit pointer
-            asm volatile("" : "+v"(lane_off));
-#pragma unroll
-            for (int i = 0; i < NB; ++i) {
-                const uint32_t blk = min((uint32_t)v[i], (uint32_t)(p.num_blocks - 1));
-                const uint64_t base = (uint64_t)blk * dma_blk_stride;
-                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(dma_kp + base + lane_off),
-                                                 LDS_PTR(kb + (16 * i + 4 * w) * KROW), 16, 0, 0);
-                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(dma_vp + base + lane_off),
-                                                 LDS_PTR(vb + (16 * i + 4 * w) * KROW), 16, 0, 0);
-            }
+            const uint32_t blk = min((uint32_t)table[first + w], (uint32_t)(p.num_blocks - 1));
+            const uint64_t base = (uint64_t)blk * dma_blk_stride;
+            // The offset is an immediate: explicit instances.  The lane offsets are made opaque once
+            // per step, so that each address stays a uniform 64-bit base plus a 32-bit lane offset
+            // (the load's scalar-base form) instead of a per-lane 64-bit pointer built with VALU adds.
+            uint32_t o0 = dma_off[0], o1 = dma_off[1], o2 = dma_off[2], o3 = dma_off[3];
+            asm volatile("" : "+v"(o0), "+v"(o1), "+v"(o2), "+v"(o3));
+            const char* kaddr = dma_kp + base;
+            const char* vaddr = dma_vp + base;
+#define AICOMP_DMA_ROWS(addr, buf, q, off)                                                                          \
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(addr + off), LDS_PTR(buf + 16 * w * KROW), 16, 1024 * q, 0);
+            AICOMP_DMA_ROWS(kaddr, kb, 0, o0) AICOMP_DMA_ROWS(kaddr, kb, 1, o1) AICOMP_DMA_ROWS(kaddr, kb, 2, o2) AICOMP_DMA_ROWS(kaddr, kb, 3, o3)
+            AICOMP_DMA_ROWS(vaddr, vb, 0, o0) AICOMP_DMA_ROWS(vaddr, vb, 1, o1) AICOMP_DMA_ROWS(vaddr, vb, 2, o2) AICOMP_DMA_ROWS(vaddr, vb, 3, o3)
+#undef AICOMP_DMA_ROWS
         } else {
             // rows at or beyond the context take the last valid row instead (finite data for
             // the masked probabilities of 0 to multiply)
             const int last = ctx - 1, last_blk = last >> 4;
+            const int bi = min(first + w, last_blk);
+            const uint32_t blk = min((uint32_t)table[bi], (uint32_t)(p.num_blocks - 1));
+            const uint64_t base = (uint64_t)blk * dma_blk_stride;
 #pragma unroll
-            for (int i = 0; i < NB; ++i) {
-                const int bi = min(first + i, last_blk);
-                const int blk = max(0, min(table[bi], p.num_blocks - 1));
-                const int64_t base = ((int64_t)blk * p.hkv + kvh) * (BS * DH * 2);
-                const int tok = min(16 * (first + i) + dma_row, last);
-                const uint32_t lane_off = (tok - 16 * bi) * (2 * DH) + ((r16 ^ dma_row) << 4);
-                __builtin_amdgcn_global_load_lds(GLOBAL_PTR((const char*)p.k_pool + base + lane_off),
-                                                 LDS_PTR(kb + (16 * i + 4 * w) * KROW), 16, 0, 0);
-                __builtin_amdgcn_global_load_lds(GLOBAL_PTR((const char*)p.v_pool + base + lane_off),
-                                                 LDS_PTR(vb + (16 * i + 4 * w) * KROW), 16, 0, 0);
+            for (int q = 0; q < 4; ++q) {
+                const int row = 4 * q + g4;
+                const int tok = min(16 * (first + w) + row, last);
+                const uint32_t off = (tok - 16 * bi) * (2 * DH) + ((r16 ^ row) << 4);
+                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(dma_kp + base + off), LDS_PTR(kb + (16 * w + 4 * q) * KROW), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(dma_vp + base + off), LDS_PTR(vb + (16 * w + 4 * q) * KROW), 16, 0, 0);
             }
         }
     };
