@@ -18,8 +18,8 @@
 //              are adjacent in the grid (one XCD's L2 serves them); the longest
 //              query tiles of a chunk are launched first.
 // K/V tiles    32 or 64 tokens per step, double-buffered in LDS, one barrier per tile.  bf16
-//              pools with D = 128 and two column groups: loaded straight into LDS
-//              (global_load_lds_dwordx4, 1 KB = four token rows per wave instruction) one tile
+//              pools and two column groups: loaded straight into LDS
+//              (global_load_lds_dwordx4, 1 KB = four or eight token rows per wave instruction) one tile
 //              ahead, rows unpadded with their 16-byte chunks XOR-swizzled by the row index.
 //              Otherwise: coalesced 16-byte loads into registers ahead of their use, written
 //              to LDS (one padded row per token; fp8 is widened to bf16 on the way).
@@ -109,7 +109,7 @@ template <int NL> struct Stage<true, NL> { uint2 k[NL], v[NL]; };
 // KT = rows of an LDS tile (KT/16 blocks): 32 with two register stages for R = 1, 64 with one stage
 // for R = 2, where the per-step work that does not scale with the tile (barrier, block lookups,
 // loop control, the running-max test) is paid half as often.
-// DMA = tiles go from the pool straight into LDS (bf16, R = 2, D = 128): no staging registers, no
+// DMA = tiles go from the pool straight into LDS (bf16 pools, R = 2): no staging registers, no
 // LDS writes by the waves.  The two buffers are separate __shared__ arrays and every read address
 // is one offset from its array, which is what lets the compiler see that a read of one buffer
 // need not wait for the loads in flight into the other; the only wait is at the barrier that
@@ -119,7 +119,7 @@ template <int NL> struct Stage<true, NL> { uint2 k[NL], v[NL]; };
 template <bool FP8, int R, int DH, bool DMA>
 __global__ void __launch_bounds__(256, (R == 1 || DH == 64) ? 3 : 2)
 paged_prefill_mfma_kernel(PrefillParams p) {
-    static_assert(!DMA || (!FP8 && R == 2 && DH == 128), "direct-to-LDS tiles: bf16, two column groups, D = 128");
+    static_assert(!DMA || (!FP8 && R == 2), "direct-to-LDS tiles: bf16 pools, two column groups");
     constexpr int KROW = DMA ? 2 * DH : 2 * DH + 16;          // LDS row stride in bytes
     constexpr int NSL = DH / 32;               // 32-element k-slots of a row (QK^T MFMAs per 16 x 16 tile)
     constexpr int NJ = DH / 16;                // 16-element output tiles (PV MFMAs per 32 tokens)
@@ -288,19 +288,27 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     // stages of 32 rows: tile t+2; one stage of 64 rows: tile t+1), so a tile's loads have the
     // time of 64 rows of arithmetic to land.
     constexpr int AHEAD = KT == 32 ? 2 : 1;
-    // Direct-to-LDS fetch of tile t: wave w brings in block w of the tile (16 token rows of 256
-    // bytes) with four instructions of 1 KB each; lane l of instruction q lands at row 4q + l/16,
-    // chunk slot l%16, and the slot holds chunk (l%16) ^ row (the XOR swizzle that keeps the
-    // operand reads free of bank conflicts without padding), so the lane reads that chunk from the
-    // pool.  One block per wave: one table entry, one base address and one LDS base per pool; the
-    // instruction's immediate offset moves the pool and the LDS address together by 1 KB per q.
+    // Direct-to-LDS fetch of tile t: wave w brings in block w of the tile (16 token rows) with
+    // 1 KB instructions, four rows of 256 bytes or eight of 128 each; lane l of instruction q lands
+    // at row RPI*q + l/CPR, chunk slot l%CPR, and the slot holds chunk (l%CPR) ^ swz(row) (the XOR
+    // swizzle that keeps the operand reads free of bank conflicts without padding), so the lane
+    // reads that chunk from the pool.  One block per wave: one table entry, one base address and
+    // one LDS base per pool; the instruction's immediate offset moves the pool and the LDS address
+    // together by 1 KB per q.
     static_assert(!DMA || NB == 4, "one block of the tile per wave");
+    constexpr int RPI = 1024 / KROW;           // token rows one 1 KB instruction lands (4 or 8)
+    constexpr int NQ = 16 / RPI;               // instructions per block and pool (4 or 2)
+    // chunk slot s of LDS row r holds chunk s ^ swz(r): sixteen consecutive rows put one chunk
+    // index into sixteen different 16-byte bank groups (256-byte rows: 16 slots; 128-byte rows:
+    // 8 slots x the two halves of the banks that even and odd rows fall into)
+    auto swz = [](int row) { return DH == 128 ? (row & 15) : ((row >> 1) & 7); };
     const uint32_t dma_blk_stride = (uint32_t)p.hkv * (BS * DH * 2);              // bytes per block, < 2^32
     const char* dma_kp = (const char*)p.k_pool + (int64_t)kvh * (BS * DH * 2);   // this KV head's slice of block 0
     const char* dma_vp = (const char*)p.v_pool + (int64_t)kvh * (BS * DH * 2);
-    uint32_t dma_off[4];                       // pool offset of this lane's chunk, less the immediate
+    const int dma_lrow = lane / CPR, dma_slot = lane % CPR;     // this lane's row and slot within 1 KB
+    uint32_t dma_off[NQ];                      // pool offset of this lane's chunk, less the immediate
 #pragma unroll
-    for (int q = 0; q < 4; ++q) dma_off[q] = g4 * (2 * DH) + ((r16 ^ g4 ^ (4 * q)) << 4);
+    for (int q = 0; q < NQ; ++q) dma_off[q] = dma_lrow * KROW + ((dma_slot ^ swz(RPI * q + dma_lrow)) << 4);
     auto fetch_dma = [&](int t, unsigned char* kb, unsigned char* vb) {
         const int first = NB * t;
         const bool tail = (t + 1) * KT > ctx || first + NB > p.max_blocks;     // workgroup-uniform
@@ -310,14 +318,15 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             // The offset is an immediate: explicit instances.  The lane offsets are made opaque once
             // per step, so that each address stays a uniform 64-bit base plus a 32-bit lane offset
             // (the load's scalar-base form) instead of a per-lane 64-bit pointer built with VALU adds.
-            uint32_t o0 = dma_off[0], o1 = dma_off[1], o2 = dma_off[2], o3 = dma_off[3];
-            asm volatile("" : "+v"(o0), "+v"(o1), "+v"(o2), "+v"(o3));
+            uint32_t o[4] = {dma_off[0], dma_off[1], dma_off[NQ > 2 ? 2 : 0], dma_off[NQ > 2 ? 3 : 1]};
+            asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]));
             const char* kaddr = dma_kp + base;
             const char* vaddr = dma_vp + base;
-#define AICOMP_DMA_ROWS(addr, buf, q, off)                                                                          \
-            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(addr + off), LDS_PTR(buf + 16 * w * KROW), 16, 1024 * q, 0);
-            AICOMP_DMA_ROWS(kaddr, kb, 0, o0) AICOMP_DMA_ROWS(kaddr, kb, 1, o1) AICOMP_DMA_ROWS(kaddr, kb, 2, o2) AICOMP_DMA_ROWS(kaddr, kb, 3, o3)
-            AICOMP_DMA_ROWS(vaddr, vb, 0, o0) AICOMP_DMA_ROWS(vaddr, vb, 1, o1) AICOMP_DMA_ROWS(vaddr, vb, 2, o2) AICOMP_DMA_ROWS(vaddr, vb, 3, o3)
+#define AICOMP_DMA_ROWS(addr, buf, q)                                                                               \
+            if constexpr (q < NQ)                                                                                   \
+                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(addr + o[q]), LDS_PTR(buf + 16 * w * KROW), 16, 1024 * q, 0);
+            AICOMP_DMA_ROWS(kaddr, kb, 0) AICOMP_DMA_ROWS(kaddr, kb, 1) AICOMP_DMA_ROWS(kaddr, kb, 2) AICOMP_DMA_ROWS(kaddr, kb, 3)
+            AICOMP_DMA_ROWS(vaddr, vb, 0) AICOMP_DMA_ROWS(vaddr, vb, 1) AICOMP_DMA_ROWS(vaddr, vb, 2) AICOMP_DMA_ROWS(vaddr, vb, 3)
 #undef AICOMP_DMA_ROWS
         } else {
             // rows at or beyond the context take the last valid row instead (finite data for
@@ -327,12 +336,12 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             const uint32_t blk = min((uint32_t)table[bi], (uint32_t)(p.num_blocks - 1));
             const uint64_t base = (uint64_t)blk * dma_blk_stride;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int row = 4 * q + g4;
+            for (int q = 0; q < NQ; ++q) {
+                const int row = RPI * q + dma_lrow;
                 const int tok = min(16 * (first + w) + row, last);
-                const uint32_t off = (tok - 16 * bi) * (2 * DH) + ((r16 ^ row) << 4);
-                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(dma_kp + base + off), LDS_PTR(kb + (16 * w + 4 * q) * KROW), 16, 0, 0);
-                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(dma_vp + base + off), LDS_PTR(vb + (16 * w + 4 * q) * KROW), 16, 0, 0);
+                const uint32_t off = (tok - 16 * bi) * KROW + ((dma_slot ^ swz(row)) << 4);
+                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(dma_kp + base + off), LDS_PTR(kb + (16 * w + RPI * q) * KROW), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(dma_vp + base + off), LDS_PTR(vb + (16 * w + RPI * q) * KROW), 16, 0, 0);
             }
         }
     };
@@ -365,8 +374,8 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             bf16x8_t a[NH];
 #pragma unroll
             for (int h = 0; h < NH; ++h)
-                if constexpr (DMA)   // chunk 4s + g4 of row 16h + prow sits at chunk slot (4s + g4) ^ prow
-                    a[h] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kb + 16 * h * KROW + prow * KROW + (((4 * s + g4) ^ prow) << 4)));
+                if constexpr (DMA)   // chunk 4s + g4 of row 16h + prow sits at chunk slot (4s + g4) ^ swz(prow)
+                    a[h] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kb + 16 * h * KROW + prow * KROW + (((4 * s + g4) ^ swz(prow)) << 4)));
                 else
                     a[h] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kb + 16 * h * KROW + rd_k + s * 64));
 #pragma unroll
@@ -471,7 +480,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             typedef short v8i16_t __attribute__((ext_vector_type(8)));
 #pragma unroll
             for (int hp = 0; hp < NH / 2; ++hp) {
-                const int voff = DMA ? 32 * hp * KROW + vrow * KROW + (((2 * j + ((r16 >> 1) & 1)) ^ vrow) << 4) + (r16 & 1) * 8
+                const int voff = DMA ? 32 * hp * KROW + vrow * KROW + (((2 * j + ((r16 >> 1) & 1)) ^ swz(vrow)) << 4) + (r16 & 1) * 8
                                      : 32 * hp * KROW + rd_v + j * 32;
                 const v4i16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(vb + voff));
                 const v4i16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(vb + (voff + 16 * KROW)));
@@ -580,7 +589,7 @@ int launch_prefill_mfma(const DecodeArgs& a, int max_q_len) {
     if (a.d == 64) {
         if (fp8 && R == 2) e = launch_prefill_variant<true, 2, 64>(p, grid, lds_bytes, a.stream);
         else if (fp8) e = launch_prefill_variant<true, 1, 64>(p, grid, lds_bytes, a.stream);
-        else if (R == 2) e = launch_prefill_variant<false, 2, 64>(p, grid, lds_bytes, a.stream);
+        else if (R == 2) e = launch_prefill_variant<false, 2, 64, true>(p, grid, 0, a.stream);    // static LDS
         else e = launch_prefill_variant<false, 1, 64>(p, grid, lds_bytes, a.stream);
     } else {
         if (fp8 && R == 2) e = launch_prefill_variant<true, 2, 128>(p, grid, lds_bytes, a.stream);

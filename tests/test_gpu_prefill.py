@@ -84,16 +84,17 @@ def test_prefill_small_ragged(device, hq, hkv):
     assert_close_attn(got, oracle(c), BF16_ATOL, BF16_RTOL, f"{hq}/{hkv}")
 
 
+@pytest.mark.parametrize("d", [128, 64])
 @pytest.mark.parametrize("ctx", [33, 63, 64, 65, 80, 127, 128, 129, 191, 193, 256, 300])
-def test_prefill_tiles_loaded_straight_into_lds(device, ctx):
-    """bf16, D = 128, >= 128 rows per chunk: the kernel whose 64-token tiles go from the pool
+def test_prefill_tiles_loaded_straight_into_lds(device, ctx, d):
+    """bf16 pools, >= 128 rows per chunk: the kernels whose 64-token tiles go from the pool
     straight into LDS.  Context lengths around the tile and block boundaries, as a fresh prompt and
     as a second chunk; every slot beyond a context is NaN (K) / Inf (V), and the table is exactly
     as wide as the longest sequence needs (a tile's block ids then run past its end)."""
     n2 = min(ctx, 40)
-    c = build_case(device, priors=[0, ctx - n2], news=[ctx, n2], hq=8, hkv=2, d=128, seed=ctx)
+    c = build_case(device, priors=[0, ctx - n2], news=[ctx, n2], hq=8, hkv=2, d=d, seed=ctx)
     got = to_f64(run(c, max_q_len=ctx))
-    assert_close_attn(got, oracle(c), BF16_ATOL, BF16_RTOL, f"ctx {ctx}")
+    assert_close_attn(got, oracle(c), BF16_ATOL, BF16_RTOL, f"ctx {ctx} D {d}")
 
 
 def test_prefill_reductions(device):
