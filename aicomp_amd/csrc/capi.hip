@@ -21,7 +21,6 @@ int launch_kv_append(const void* key, const void* value, int64_t token_stride, i
                      int d, int bs, int64_t num_blocks, int in_dtype, int pool_dtype,
                      const float* k_scale, const float* v_scale, hipStream_t stream);
 
-struct PrefillArgs;
 bool prefill_mfma_supported(const DecodeArgs& a, int max_q_len);
 int launch_prefill_mfma(const DecodeArgs& a, int max_q_len);
 
@@ -228,6 +227,10 @@ static int decode_impl(void* out, const void* query, const void* new_key, const 
     a.partition_size = partition_size;
     a.num_parts = resolve_parts(batch, num_kv_heads, block_size, max_blocks_per_seq, a.partition_size);
     a.stream = (hipStream_t)stream;
+    // the matrix-core kernels append the new rows themselves when they can read them 16 bytes at a time
+    const bool injectable = fused && q_dtype == AICOMP_KV_BF16 && kv_token_stride % 8 == 0 &&
+                            kv_head_stride % 8 == 0 && (uintptr_t)new_key % 16 == 0 &&
+                            (uintptr_t)new_value % 16 == 0;
     if (partition_size == 0 && decode_streamk_supported(a)) {
         // balanced schedule: equal tile counts per wave, merged by a second kernel
         const size_t need = decode_streamk_workspace_bytes(a.rows, a.hq, a.hkv, a.d);
@@ -236,10 +239,7 @@ static int decode_impl(void* out, const void* query, const void* new_key, const 
                        workspace ? workspace_bytes : (size_t)0);
         AICOMP_REQUIRE((uintptr_t)workspace % 16 == 0, AICOMP_KV_EINVAL,
                        "%s: workspace must be 16-byte aligned", who);
-        // the kernel appends the new rows itself when it can read them 16 bytes at a time
-        const bool in_kernel = fused && q_dtype == AICOMP_KV_BF16 && kv_token_stride % 8 == 0 &&
-                               kv_head_stride % 8 == 0 && (uintptr_t)new_key % 16 == 0 &&
-                               (uintptr_t)new_value % 16 == 0;
+        const bool in_kernel = injectable;
         if (fused && !in_kernel) {
             rc = launch_kv_append_last(new_key, new_value, kv_token_stride, kv_head_stride, k_pool, v_pool,
                                        block_table, block_table_stride, context_lens, batch,
@@ -253,11 +253,8 @@ static int decode_impl(void* out, const void* query, const void* new_key, const 
         }
         return launch_decode_streamk(a, workspace);
     }
-    // the grid-scheduled matrix-core kernel appends the new rows itself under the same conditions
     const bool mfma = decode_mfma_supported(a);
-    const bool in_kernel = fused && mfma && q_dtype == AICOMP_KV_BF16 && kv_token_stride % 8 == 0 &&
-                           kv_head_stride % 8 == 0 && (uintptr_t)new_key % 16 == 0 &&
-                           (uintptr_t)new_value % 16 == 0;
+    const bool in_kernel = injectable && mfma;
     if (in_kernel) {
         a.new_key = new_key; a.new_value = new_value;
         a.new_token_stride = kv_token_stride; a.new_head_stride = kv_head_stride;
