@@ -61,6 +61,7 @@ struct PrefillParams {
     const int32_t* cu_q_lens;
     int hq, hkv, group, gpack, max_blocks;
     int num_blocks;
+    int num_cus;                       // CUs of the device (0: keep the grid order)
     float qk_mul;
     const float* k_scale;
     const float* v_scale;
@@ -131,26 +132,90 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     constexpr int NL = KT / RPL;               // loads per tile and pool
     typedef Stage<FP8, NL> StageT;
     // Grid: x = head group (fastest: the workgroups of one KV head land on one XCD and share its
-    // L2 copy of that head's K/V), y = sequence, z = query tile, longest first (the last tile of a
-    // chunk sees the most keys, so it is started first).  Sequence before tile: workgroups that
-    // are resident together then come from different chunks, which evens out what a CU is given
-    // (measured 102 us against 107 us with the tile index in y on four chunks of 512).
+    // L2 copy of that head's K/V); (y, z) number the (sequence, query tile) items.
     constexpr int TT = KT;                     // tokens per LDS tile
     constexpr int CR = 16;                     // query rows per 16-column group
     constexpr int WROWS = CR * R;              // rows per wave
-    const int seq = blockIdx.y;
     const int hgroup = blockIdx.x;
-    const int qtile = gridDim.z - 1 - blockIdx.z;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r16 = lane & 15, g4 = lane >> 4;
+    const int pos_per_wg = 4 * WROWS / p.gpack;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [2][K tile | V tile]
+    // Direct-to-LDS tiles: four separate arrays, so that the compiler can tell a read of one
+    // buffer from the loads in flight into the other.
+    __shared__ __attribute__((aligned(16))) unsigned char dma_k0[DMA ? TILE_BYTES : 16];
+    __shared__ __attribute__((aligned(16))) unsigned char dma_v0[DMA ? TILE_BYTES : 16];
+    __shared__ __attribute__((aligned(16))) unsigned char dma_k1[DMA ? TILE_BYTES : 16];
+    __shared__ __attribute__((aligned(16))) unsigned char dma_v1[DMA ? TILE_BYTES : 16];
+
+    // Which item this workgroup takes.  Workgroups are dispatched in grid order, the first
+    // num_cus of them one per CU, the next num_cus beside them, the rest as places free up; an
+    // item costs as many tile steps as its last row has keys, and chunks with different prior
+    // contexts differ several-fold.  For 2 to 16 chunks and up to 256 items every workgroup ranks
+    // the items by cost (same inputs, same answer everywhere) and takes the item whose rank is its
+    // own place in the dispatch order, odd rounds of num_cus reversed: the two workgroups that share
+    // a CU from the start are then a long item and a short one, and later places are handed out
+    // longest first.  An item's rank comes in closed form from the other chunks' lengths (its
+    // cost c, then per chunk the number of tiles costing >= c and >= c + 1), so the work is per
+    // chunk, not per item.  Other grids keep the grid order, longest tile of every chunk first.
+    int seq = blockIdx.y, qtile = gridDim.z - 1 - blockIdx.z;
+    const int nseq = gridDim.y, ntile = gridDim.z, items = nseq * ntile;
+    if (p.num_cus > 0 && nseq > 1 && nseq <= 16 && items <= 256) {     // workgroup-uniform
+        int* scratch = (int*)(DMA ? dma_k0 : lds);                     // the tile buffers are still unused
+        if (tid < nseq) {
+            const int n_t = p.cu_q_lens[tid + 1] - p.cu_q_lens[tid];
+            const int ctx_t = min(p.context_lens[tid], p.max_blocks * BS);
+            scratch[4 * tid] = ctx_t;
+            scratch[4 * tid + 1] = ctx_t - n_t;
+            scratch[4 * tid + 2] = (n_t > 0 && ctx_t >= n_t) ? (n_t + pos_per_wg - 1) / pos_per_wg : 0;   // tiles with work
+        }
+        __syncthreads();
+        // this workgroup's place among the items, and the rank it takes
+        const int place = blockIdx.y + nseq * blockIdx.z;
+        int want = place;
+        const int per_round = p.num_cus / (int)gridDim.x;
+        if (per_round > 0 && p.num_cus % (int)gridDim.x == 0) {
+            const int round = place / per_round, pos = place % per_round;
+            const int cnt = min(per_round, items - round * per_round);
+            if (round & 1) want = round * per_round + (cnt - 1 - pos);
+        }
+        const int shift = __builtin_ctz(pos_per_wg);                    // a power of two
+        // tiles of a chunk (context, prior, tiles) that cost at least c steps (c >= 1)
+        auto count_ge = [&](int ctx_s, int prior_s, int tiles_s, int c) {
+            const int x = (c - 1) * KT;
+            if (tiles_s == 0 || ctx_s <= x) return 0;
+            return max(0, tiles_s - (x < prior_s ? 0 : (x - prior_s) >> shift));
+        };
+        if (tid < items) {
+            const int s_t = tid / ntile, q_t = tid - s_t * ntile;
+            const int ctx_t = scratch[4 * s_t], prior_t = scratch[4 * s_t + 1], tiles_t = scratch[4 * s_t + 2];
+            const bool work = q_t < tiles_t;
+            const int c = work ? (min(ctx_t, prior_t + (q_t + 1) * pos_per_wg) + KT - 1) / KT : 0;
+            int dearer = 0, equal_before = 0, all_work = 0, idle_before = 0;
+            for (int s2 = 0; s2 < nseq; ++s2) {
+                const int ctx2 = scratch[4 * s2], prior2 = scratch[4 * s2 + 1], tiles2 = scratch[4 * s2 + 2];
+                const int ge1 = count_ge(ctx2, prior2, tiles2, c + 1), ge0 = count_ge(ctx2, prior2, tiles2, max(c, 1));
+                dearer += ge1;
+                if (s2 < s_t) { equal_before += ge0 - ge1; idle_before += ntile - tiles2; }
+                if (s2 == s_t) equal_before += q_t - (tiles2 - ge0);    // costs do not fall along a chunk
+                all_work += tiles2;
+            }
+            const int rank = work ? dearer + equal_before : all_work + idle_before + (q_t - tiles_t);
+            if (rank == want) { scratch[64] = s_t; scratch[65] = q_t; }
+        }
+        __syncthreads();
+        seq = __builtin_amdgcn_readfirstlane(scratch[64]);
+        qtile = __builtin_amdgcn_readfirstlane(scratch[65]);
+        __syncthreads();                       // before the first tile is written over the scratch
+    }
 
     const int q_begin = p.cu_q_lens[seq];
     const int n = p.cu_q_lens[seq + 1] - q_begin;
     const int ctx = min(p.context_lens[seq], p.max_blocks * BS);
     const int prior = ctx - n;
-    const int pos_per_wg = 4 * WROWS / p.gpack;
     const int q0 = qtile * pos_per_wg;
     if (q0 >= n || n <= 0 || prior < 0) return;
 
@@ -171,14 +236,6 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     const int wave_kv_min = prior + q0 + (WROWS * w) / p.gpack;    // smallest qabs in the wave (if valid)
     const int kv_end = min(ctx, prior + q0 + pos_per_wg);
     const int ntiles = (kv_end + TT - 1) / TT;
-
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [2][K tile | V tile]
-    // Direct-to-LDS tiles: four separate arrays, so that the compiler can tell a read of one
-    // buffer from the loads in flight into the other.
-    __shared__ __attribute__((aligned(16))) unsigned char dma_k0[DMA ? TILE_BYTES : 16];
-    __shared__ __attribute__((aligned(16))) unsigned char dma_v0[DMA ? TILE_BYTES : 16];
-    __shared__ __attribute__((aligned(16))) unsigned char dma_k1[DMA ? TILE_BYTES : 16];
-    __shared__ __attribute__((aligned(16))) unsigned char dma_v1[DMA ? TILE_BYTES : 16];
 
     // Q as the B operand: column = this lane's row, k-slots = dims 32s + 8*g4 ..
     bf16x8_t qf[R][NSL];
@@ -574,6 +631,19 @@ int launch_prefill_mfma(const DecodeArgs& a, int max_q_len) {
     AICOMP_REQUIRE(a.num_blocks <= INT32_MAX, AICOMP_KV_EINVAL, "paged_prefill_attn: num_blocks too large");
     p.num_blocks = (int)a.num_blocks;
     p.gpack = (16 % p.group == 0) ? p.group : 1;      // heads of one KV head packed per position
+    // CU count of the first device used (every GPU of a node is the same part); 0 if unknown, which
+    // only turns the cost-ranked item order off
+    static std::atomic<int> cached_cus{-1};
+    int num_cus = cached_cus.load(std::memory_order_relaxed);
+    if (num_cus < 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 0)
+            n = 0;
+        num_cus = n;
+        cached_cus.store(n, std::memory_order_relaxed);
+    }
+    p.num_cus = num_cus;
     p.qk_mul = a.scale * LOG2E;
     p.k_scale = a.k_scale; p.v_scale = a.v_scale;
     // two column groups per wave (128 rows per workgroup) once a chunk has that many rows

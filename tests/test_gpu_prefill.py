@@ -97,6 +97,26 @@ def test_prefill_tiles_loaded_straight_into_lds(device, ctx, d):
     assert_close_attn(got, oracle(c), BF16_ATOL, BF16_RTOL, f"ctx {ctx} D {d}")
 
 
+@pytest.mark.parametrize("d", [128, 64])
+def test_prefill_items_taken_in_cost_order(device, d):
+    """2 to 16 chunks: workgroups take (chunk, query tile) items by rank of cost, not by grid
+    position.  Chunks of very different prior context and length, one of them empty, equal costs
+    across chunks, more tiles in the grid than most chunks have: every row must still be computed
+    exactly once (the output starts as NaN)."""
+    priors = [1900, 0, 300, 300, 77, 1024, 0, 512, 5]
+    news = [512, 512, 40, 40, 0, 130, 1, 200, 333]
+    c = build_case(device, priors=priors, news=news, hq=8, hkv=2, d=d, seed=5)
+    got = run(c, max_q_len=512)
+    assert torch.isfinite(got.float()).all()
+    assert_close_attn(to_f64(got), oracle(c), BF16_ATOL, BF16_RTOL, f"cost order D {d}")
+    # sixteen chunks, and seventeen (which keeps the grid order)
+    for nseq in (16, 17):
+        pr = [(i * 211) % 700 for i in range(nseq)]
+        nw = [32 + (i * 37) % 150 for i in range(nseq)]
+        c = build_case(device, priors=pr, news=nw, hq=8, hkv=2, d=d, seed=nseq)
+        assert_close_attn(to_f64(run(c, max_q_len=max(nw))), oracle(c), BF16_ATOL, BF16_RTOL, f"{nseq} chunks D {d}")
+
+
 def test_prefill_reductions(device):
     c = build_case(device, priors=[0, 300], news=[96, 1], hq=8, hkv=2, d=128, poison=False)
     got = run(c)
