@@ -170,7 +170,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             const int ctx_t = min(p.context_lens[tid], p.max_blocks * BS);
             scratch[4 * tid] = ctx_t;
             scratch[4 * tid + 1] = ctx_t - n_t;
-            scratch[4 * tid + 2] = (n_t > 0 && ctx_t >= n_t) ? (n_t + pos_per_wg - 1) / pos_per_wg : 0;   // tiles with work
+            scratch[4 * tid + 2] = (n_t > 0 && ctx_t >= n_t) ? min(ntile, (n_t + pos_per_wg - 1) / pos_per_wg) : 0;   // tiles with work
         }
         __syncthreads();
         // this workgroup's place among the items, and the rank it takes
