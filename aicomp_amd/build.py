@@ -54,7 +54,8 @@ def build_host_example(verbose: bool = True) -> str:
     torch): the boundary as a C or C++ host sees it."""
     root = os.path.dirname(HERE)
     src, exe = os.path.join(root, "tests", "cabi_host.cpp"), os.path.join(root, "tests", "cabi_host")
-    cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-I" + os.path.join(root, "include"), src,
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-I" + os.path.join(root, "include"), src,
            "-L" + HERE, "-laicomp_kv", "-Wl,-rpath,$ORIGIN/../aicomp_amd", "-o", exe]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
