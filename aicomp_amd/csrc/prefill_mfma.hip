@@ -407,7 +407,12 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         const unsigned char* kb;
         const unsigned char* vb;
         if constexpr (DMA) {
-            __syncthreads();      // tile t has landed (own loads waited for, then everyone's); tile t-1 is no longer read
+            // Tile t has landed once every wave has waited for its own direct-to-LDS loads and
+            // then met the others.  The wait is explicit: the compiler only waits for such loads
+            // before this wave's own aliasing LDS reads, which says nothing about the other waves'
+            // loads, and on the loop's back edge it was seen to emit no wait at all.
+            __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0)
+            __syncthreads();      // also: tile t-1 is no longer read by anyone
             if (t + 1 < ntiles) fetch_dma(t + 1, kn, vn);
             kb = kb_; vb = vb_;
         } else {
