@@ -15,12 +15,15 @@
 //              head packed per position, the rows are consecutive positions x G
 //              heads, so every K/V tile staged in LDS serves the whole GQA group.
 //              Groups that do not divide 16 use gpack = 1.  Workgroups of one KV head
-//              are adjacent in the grid (one XCD's L2 serves them); the longest
-//              query tiles of a chunk are launched first.
+//              are adjacent in the grid (one XCD's L2 serves them).  With 2 to 16 chunks the
+//              workgroups take their (chunk, query tile) items in order of cost, a long item
+//              and a short one side by side on a CU; otherwise the longest query tiles of
+//              every chunk are launched first.
 // K/V tiles    32 or 64 tokens per step, double-buffered in LDS, one barrier per tile.  bf16
 //              pools and two column groups: loaded straight into LDS
-//              (global_load_lds_dwordx4, 1 KB = four or eight token rows per wave instruction) one tile
-//              ahead, rows unpadded with their 16-byte chunks XOR-swizzled by the row index.
+//              (global_load_lds_dwordx4, 1 KB = four or eight token rows per wave
+//              instruction) one tile ahead, rows unpadded with their 16-byte chunks
+//              XOR-swizzled by the row index.
 //              Otherwise: coalesced 16-byte loads into registers ahead of their use, written
 //              to LDS (one padded row per token; fp8 is widened to bf16 on the way).
 // head_dim     128 or 64, one instantiation each.
@@ -29,10 +32,11 @@
 //              (v_mfma_f32_16x16x32_bf16); online softmax per column on the raw
 //              scores with a lazily moved max: the exponentials are taken against the current
 //              max and their sum tells whether it has to move (then, rarely, the row max is
-//              found with two lane swaps and the exponentials are redone); O^T += V^T P^T with the V^T operand read out of the row-major
-//              V tile by gfx950's transposing LDS read (ds_read_b64_tr_b16), in the token
-//              order the QK product was laid out in, so P never leaves its lane.  With two
-//              column groups every LDS operand read feeds two MFMAs.
+//              found with two lane swaps and the exponentials are redone); O^T += V^T P^T
+//              with the V^T operand read out of the row-major V tile by gfx950's transposing
+//              LDS read (ds_read_b64_tr_b16), in the token order the QK product was laid out
+//              in, so P never leaves its lane.  With two column groups every LDS operand
+//              read feeds two MFMAs.
 #include "common.h"
 
 #include <atomic>
@@ -105,16 +109,17 @@ template <int NL> struct Stage<true, NL> { uint2 k[NL], v[NL]; };
 // R = 16-row column groups per wave (1 or 2).  With R = 2 every K and V operand read from LDS
 // (and every V permute) feeds two MFMAs, and the two groups' softmax chains are independent, so
 // LDS traffic and permute work per flop halve and the scheduler has two chains to interleave.
-// DH = head_dim (128 or 64).  An LDS row is one token: 2*DH bytes plus 16 bytes of padding, so that
-// the sixteen rows of an operand read start in different banks (272 B: 4 banks apart; 144 B: 36).
+// DH = head_dim (128 or 64).  An LDS row is one token: 2*DH bytes plus, in the register-staged
+// variants, 16 bytes of padding, so that the sixteen rows of an operand read start in different
+// banks (272 B: 4 banks apart; 144 B: 36).
 // KT = rows of an LDS tile (KT/16 blocks): 32 with two register stages for R = 1, 64 with one stage
 // for R = 2, where the per-step work that does not scale with the tile (barrier, block lookups,
 // loop control, the running-max test) is paid half as often.
 // DMA = tiles go from the pool straight into LDS (bf16 pools, R = 2): no staging registers, no
 // LDS writes by the waves.  The two buffers are separate __shared__ arrays and every read address
 // is one offset from its array, which is what lets the compiler see that a read of one buffer
-// need not wait for the loads in flight into the other; the only wait is at the barrier that
-// opens a step, for the loads issued one step earlier.
+// need not wait for the loads in flight into the other; the only wait is the explicit one at the
+// barrier that opens a step, for the loads issued one step earlier.
 #define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 template <bool FP8, int R, int DH, bool DMA>
