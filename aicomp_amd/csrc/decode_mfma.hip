@@ -595,10 +595,6 @@ __device__ __forceinline__ int sk_tiles(int len, int max_blocks) {
     return (len + TILE - 1) / TILE;
 }
 
-// wave that owns global tile g when N tiles are dealt to W waves as [i*N/W, (i+1)*N/W)
-__device__ __forceinline__ int sk_wave_of(int64_t g, int64_t N, int W) {
-    return (int)(((g + 1) * W - 1) / N);
-}
 
 template <bool FP8>
 __global__ void __launch_bounds__(256, 1)     // one workgroup per CU: a wave may use the whole register file
