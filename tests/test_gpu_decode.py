@@ -408,3 +408,53 @@ def test_fused_append_in_the_grid_kernel_edge_positions(device, d, kv, ps):
     assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
     want = oracle_decode(w, ctx=ctx.cpu().numpy())
     assert_close_attn(to_f64(out), want, BF16_ATOL, BF16_RTOL, f"grid fused append D={d}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("hkv,group", [(8, 4), (3, 2), (16, 1)])
+def test_balanced_schedule_records_the_parts_the_host_model_predicts(hkv, group):
+    """The main kernel of the balanced schedule tells the merge kernel, per (sequence, KV head)
+    row, which of the head's parts hold the row's first and last tile.  tests/test_decode_schedule.py
+    models the schedule on the host and checks its invariants (coverage, distinct slots, bounds);
+    this test ties that model to the kernel by reading the record back from the caller's scratch."""
+    import math
+    from aicomp_amd import ops
+    from test_decode_schedule import SK_MAX_WAVES, schedule, tiles_of
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(11 + hkv)
+    B, D, hq = 37, 128, hkv * group
+    lens = torch.randint(1, 3000, (B,), generator=g).tolist()
+    lens[3] = 0; lens[4] = 0; lens[20] = 1; lens[36] = 33
+    need = [max(1, math.ceil(c / 16)) for c in lens]
+    max_blocks = max(need)
+    nb = sum(need) + 1
+    perm = torch.randperm(nb, generator=g)
+    table = torch.zeros(B, max_blocks, dtype=torch.int32)
+    cur = 0
+    for s, n in enumerate(need):
+        table[s, :n] = perm[cur:cur + n].to(torch.int32); cur += n
+    k = torch.randn(nb, hkv, 16, D, generator=g).to(torch.bfloat16).to(dev)
+    v = torch.randn(nb, hkv, 16, D, generator=g).to(torch.bfloat16).to(dev)
+    q = torch.randn(B, hq, D, generator=g).to(torch.bfloat16).to(dev)
+    out = torch.empty_like(q)
+    cl = torch.tensor(lens, dtype=torch.int32, device=dev)
+    nbytes = ops.decode_workspace_bytes(B, hq, hkv, D, 16, max_blocks, q.dtype, k.dtype)
+    ws = torch.full((nbytes,), 0xA5, dtype=torch.uint8, device=dev)
+    ops.paged_decode_attn(out, q, k, v, table.to(dev), cl, 1 / math.sqrt(D), None, None, workspace=ws)
+    torch.cuda.synchronize()
+    slots = SK_MAX_WAVES + B * hkv
+    off = slots * group * D + slots * group * 2                 # partial outputs, then (max, sum) pairs
+    assert nbytes >= (off + B * hkv * 2) * 4
+    rec = ws.view(torch.int32)[off:off + B * hkv * 2].reshape(B, hkv, 2).cpu()
+    num_waves = 4 * torch.cuda.get_device_properties(0).multi_processor_count
+    segs, _ = schedule(lens, hkv, num_waves, max_blocks)
+    first, last = {}, {}
+    for kvh, part, seq, t, nt, slot in segs:
+        if t == 0:
+            first[(seq, kvh)] = part
+        if t + nt == tiles_of(lens[seq], max_blocks):
+            last[(seq, kvh)] = part
+    for s in range(B):
+        for h in range(hkv):
+            if lens[s] > 0:
+                assert (int(rec[s, h, 0]), int(rec[s, h, 1])) == (first[(s, h)], last[(s, h)]), (s, h)
