@@ -18,6 +18,7 @@ SYMBOLS = (
     "aicomp_kv_append",
     "aicomp_paged_decode_attn",
     "aicomp_paged_decode_attn_append",
+    "aicomp_paged_decode_attn_append_static",
     "aicomp_paged_decode_workspace_bytes",
     "aicomp_paged_decode_partition_size",
     "aicomp_paged_prefill_attn",
@@ -51,6 +52,10 @@ def _declare(lib: C.CDLL) -> None:
     lib.aicomp_paged_decode_attn_append.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp, i64, vp, i32, i32,
                                                     i32, i32, i32, i32, i64, f32, i32, i32, vp, vp, i32,
                                                     vp, sz, vp]
+    lib.aicomp_paged_decode_attn_append_static.restype = i32
+    lib.aicomp_paged_decode_attn_append_static.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp, i64, vp, i32,
+                                                           i32, i32, i32, i32, i32, i64, f32, i32, i32, vp,
+                                                           vp, i32, vp]
     lib.aicomp_paged_decode_workspace_bytes.restype = sz
     lib.aicomp_paged_decode_workspace_bytes.argtypes = [i32] * 9
     lib.aicomp_paged_decode_partition_size.restype = i32

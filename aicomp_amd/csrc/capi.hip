@@ -5,6 +5,13 @@
 
 #include <string.h>
 
+#include <atomic>
+
+// Split-K scratch of aicomp_paged_decode_attn_append_static: device memory that belongs to the
+// loaded library, one copy per GPU, held until the process ends.  In host code this name is only
+// a handle for hipGetSymbolAddress: the address a kernel may use is what that call returns.
+static __device__ __align__(256) unsigned char scratch[AICOMP_KV_STATIC_SCRATCH_BYTES];
+
 namespace aicomp {
 
 static thread_local char g_err[512] = "";
@@ -310,6 +317,58 @@ int aicomp_paged_decode_attn_append(void* out, const void* query, const void* ne
                        head_dim, block_size, max_blocks_per_seq, num_blocks, scale, q_dtype, kv_dtype,
                        k_scale, v_scale, partition_size, workspace, workspace_bytes, stream,
                        "paged_decode_attn_append");
+}
+
+// Device address of `scratch` on the current device, looked up once per device.
+static int static_scratch(void** ptr, const char* who) {
+    constexpr int MAX_DEVICES = 64;
+    static std::atomic<void*> per_device[MAX_DEVICES];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+        set_error("%s: cannot identify the current device (%d)", who, dev);
+        return AICOMP_KV_EHIP;
+    }
+    void* p = per_device[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr) {
+            set_error("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", who, dev,
+                      hipGetErrorString(e));
+            return AICOMP_KV_EHIP;
+        }
+        per_device[dev].store(p, std::memory_order_release);     // racing threads store the same address
+    }
+    *ptr = p;
+    return AICOMP_KV_OK;
+}
+
+int aicomp_paged_decode_attn_append_static(void* out, const void* query, const void* new_key,
+                                           const void* new_value, int64_t kv_token_stride,
+                                           int64_t kv_head_stride, void* k_pool, void* v_pool,
+                                           const int32_t* block_table, int64_t block_table_stride,
+                                           const int32_t* context_lens, int batch, int num_q_heads,
+                                           int num_kv_heads, int head_dim, int block_size,
+                                           int max_blocks_per_seq, int64_t num_blocks, float scale,
+                                           int q_dtype, int kv_dtype, const float* k_scale,
+                                           const float* v_scale, int partition_size, void* stream) {
+    const char* who = "paged_decode_attn_append_static";
+    AICOMP_REQUIRE(batch <= 0 || (new_key && new_value), AICOMP_KV_EINVAL, "%s: null new_key / new_value", who);
+    const size_t need = aicomp_paged_decode_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim,
+                                                            block_size, max_blocks_per_seq, q_dtype,
+                                                            kv_dtype, partition_size);
+    AICOMP_REQUIRE(need <= (size_t)AICOMP_KV_STATIC_SCRATCH_BYTES, AICOMP_KV_EWORKSPACE,
+                   "%s: this shape needs %zu bytes of split-K scratch, the built-in scratch holds %zu; "
+                   "use aicomp_paged_decode_attn_append with a workspace of the caller's", who, need,
+                   (size_t)AICOMP_KV_STATIC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    if (need > 0) {
+        const int rc = static_scratch(&ws, who);
+        if (rc) return rc;
+    }
+    return decode_impl(out, query, new_key, new_value, kv_token_stride, kv_head_stride, k_pool, v_pool,
+                       block_table, block_table_stride, context_lens, batch, num_q_heads, num_kv_heads,
+                       head_dim, block_size, max_blocks_per_seq, num_blocks, scale, q_dtype, kv_dtype,
+                       k_scale, v_scale, partition_size, ws, need, stream, who);
 }
 
 int aicomp_paged_prefill_attn(void* out, const void* query, const void* k_pool, const void* v_pool,

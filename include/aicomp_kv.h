@@ -137,6 +137,36 @@ int aicomp_paged_decode_attn_append(void* out, const void* query,
                                     void* workspace, size_t workspace_bytes,
                                     void* stream);
 
+/*
+ * aicomp_paged_decode_attn_append for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments, results and bit patterns as
+ * aicomp_paged_decode_attn_append, without the workspace pair: the split-K partials go to a
+ * scratch array of AICOMP_KV_STATIC_SCRATCH_BYTES that is part of the loaded library (every GPU
+ * the library runs on holds its own copy until the process ends).  The call allocates, frees and
+ * clears nothing (no partial is read that the same call did not write, so nothing has to start
+ * at zero).  The first call on a device looks the array's address up (hipGetSymbolAddress); make
+ * that call outside graph capture, with the device of the pointers current.
+ *
+ * A shape whose aicomp_paged_decode_workspace_bytes() exceeds AICOMP_KV_STATIC_SCRATCH_BYTES is
+ * refused with AICOMP_KV_EWORKSPACE (32 MiB covers batch 128 at 64 / 8 heads, head_dim 128).
+ * All calls on one GPU share that GPU's array: calls that may overlap in time (different
+ * streams, or several host threads on one device) race on the partials; serialise them or use
+ * aicomp_paged_decode_attn_append with one workspace per stream.
+ */
+#define AICOMP_KV_STATIC_SCRATCH_BYTES (32u << 20)
+int aicomp_paged_decode_attn_append_static(void* out, const void* query,
+                                           const void* new_key, const void* new_value,
+                                           int64_t kv_token_stride, int64_t kv_head_stride,
+                                           void* k_pool, void* v_pool,
+                                           const int32_t* block_table, int64_t block_table_stride,
+                                           const int32_t* context_lens,
+                                           int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                                           int block_size, int max_blocks_per_seq, int64_t num_blocks,
+                                           float scale, int q_dtype, int kv_dtype,
+                                           const float* k_scale, const float* v_scale,
+                                           int partition_size, void* stream);
+
 size_t aicomp_paged_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads,
                                            int head_dim, int block_size,
                                            int max_blocks_per_seq, int q_dtype, int kv_dtype,
