@@ -451,7 +451,12 @@ paged_decode_mfma_kernel(MfmaParams p) {
         // the sequence's newest token lives in this tile (bb still holds its blocks: the last lookup
         // above was for this wave's final tile)
         if (p.new_key != nullptr && end == len && tile_start < len && tile_start + TT >= len) {
-            inject_new_row_grid<FP8, PAIR>(kr, vr, p, seq, kvh, lane, tile_start, len, bb);
+            // Same rule as the separate one-token append: the row is stored only where the table names a
+            // block of the pool and the length fits the table; otherwise the call leaves the pools alone
+            // (and attends over what the clamped table entry holds, like the unfused sequence of calls).
+            const int raw_blk = __builtin_amdgcn_readlane(tab, BPT * tt + ((len - 1 - tile_start) >> 4) - tab_first);
+            if (p.context_lens[seq] == len && raw_blk >= 0 && raw_blk < p.num_blocks)
+                inject_new_row_grid<FP8, PAIR>(kr, vr, p, seq, kvh, lane, tile_start, len, bb);
         }
         if (tile_start + TT > end)
             process_tile<FP8, false, true, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
@@ -766,7 +771,12 @@ streamk_decode_kernel(StreamKParams p) {
         const int tile_start = (t + k) * TILE;
         if (p.new_key != nullptr && t + k == row_tiles - 1) {       // the row's newest token lives here
             tile_blocks(k, b0, b1);
-            inject_new_row<FP8>(kr, vr, p, seq, kvh, lane, tile_start, len, b0, b1);
+            // Same rule as the separate one-token append: the row is stored only where the table names a
+            // block of the pool and the length fits the table; otherwise the call leaves the pools alone
+            // (and attends over what the clamped table entry holds, like the unfused sequence of calls).
+            const int raw_blk = __builtin_amdgcn_readlane(tab, 2 * k + ((len - 1 - tile_start) >> 4) - tab_first);
+            if (p.context_lens[seq] == len && raw_blk >= 0 && raw_blk < p.num_blocks)
+                inject_new_row<FP8>(kr, vr, p, seq, kvh, lane, tile_start, len, b0, b1);
         }
         // The segment's last tile always runs the masked body (a full tile simply masks nothing):
         // one prefetching call site, so the prefetched registers need no merging afterwards.

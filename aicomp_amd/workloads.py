@@ -14,7 +14,7 @@ from __future__ import annotations
 
 import math
 from dataclasses import dataclass, field
-from typing import Dict, List, Optional
+from typing import Dict, List, Optional, Sequence
 
 import torch
 
@@ -136,6 +136,50 @@ def _context_lengths(shape: Shape, g: torch.Generator) -> List[int]:
     return L.clamp(shape.ctx_lo, shape.ctx_hi).long().tolist()
 
 
+def _fp8_source_chunks(pool_shape, dev: torch.device, seed: int):
+    """The N(0,1) data an fp8 pool is quantised from, a few thousand blocks at a time:
+    yields (first block, blocks, K chunk, V chunk) in float32, the same values on every pass."""
+    pool_blocks, hkv, bs, d = pool_shape
+    step = max(1, (1 << 24) // (hkv * bs * d))
+    sg = torch.Generator(device=dev).manual_seed(seed + 2)
+    for i in range(0, pool_blocks, step):
+        m = min(step, pool_blocks - i)
+        kk = torch.randn(m, hkv, bs, d, generator=sg, device=dev)
+        vv = torch.randn(m, hkv, bs, d, generator=sg, device=dev)
+        yield i, m, kk, vv
+
+
+def unquantised_context(w: "Workload", seqs: Sequence[int], seed: int = 0):
+    """For an fp8 workload built by ``make_workload(..., seed=seed)``: the float32 K and V rows,
+    before quantisation, of the given sequences' contexts, the step's new token included
+    (``[(K [L, Hkv, D], V [L, Hkv, D]), ...]`` on the workload's device).  What the fp8 path's
+    error against the unquantised model is measured from."""
+    if w.k_pool.dtype != torch.float8_e4m3fn:
+        raise ValueError("unquantised_context is for fp8 workloads")
+    dev, bs = w.k_pool.device, w.shape.block_size
+    tables = w.block_table.cpu()
+    want = []
+    for s in seqs:
+        L = w.ctx_list[s]
+        t = torch.arange(L)
+        want.append((tables[s, t // bs].long(), t % bs))
+    outs = [(torch.empty(w.ctx_list[s], w.k_pool.shape[1], w.k_pool.shape[3], device=dev),
+             torch.empty(w.ctx_list[s], w.k_pool.shape[1], w.k_pool.shape[3], device=dev)) for s in seqs]
+    for i, m, kk, vv in _fp8_source_chunks(tuple(w.k_pool.shape), dev, seed):
+        for (blk, off), (ko, vo) in zip(want, outs):
+            hit = ((blk >= i) & (blk < i + m)).nonzero().flatten()
+            if hit.numel():
+                b, o = (blk[hit] - i).to(dev), off[hit].to(dev)
+                ko[hit.to(dev)] = kk[b, :, o, :]
+                vo[hit.to(dev)] = vv[b, :, o, :]
+    cu = w.cu_q_lens.cpu().tolist()
+    for s, (ko, vo) in zip(seqs, outs):               # the step's own rows come from new_key / new_value
+        n = w.new_list[s]
+        ko[w.ctx_list[s] - n:] = w.new_key[cu[s]:cu[s] + n].float()
+        vo[w.ctx_list[s] - n:] = w.new_value[cu[s]:cu[s] + n].float()
+    return outs
+
+
 def make_workload(name: str, device="cpu", seed: int = 0, shape: Optional[Shape] = None) -> Workload:
     """Build one step of the named workload.
 
@@ -204,23 +248,14 @@ def make_workload(name: str, device="cpu", seed: int = 0, shape: Optional[Shape]
         v_pool = torch.empty(pool_shape, dtype=shape.kv_dtype, device=dev)
         amax_k = torch.zeros(hkv, device=dev)
         amax_v = torch.zeros(hkv, device=dev)
-        step = max(1, (1 << 24) // (hkv * bs * d))
-        sg = torch.Generator(device=dev).manual_seed(seed + 2)
-        for i in range(0, pool_blocks, step):
-            m = min(step, pool_blocks - i)
-            amax_k = torch.maximum(amax_k, torch.randn(m, hkv, bs, d, generator=sg, device=dev)
-                                   .abs().amax(dim=(0, 2, 3)))
-            amax_v = torch.maximum(amax_v, torch.randn(m, hkv, bs, d, generator=sg, device=dev)
-                                   .abs().amax(dim=(0, 2, 3)))
+        for i, m, kk, vv in _fp8_source_chunks(pool_shape, dev, seed):
+            amax_k = torch.maximum(amax_k, kk.abs().amax(dim=(0, 2, 3)))
+            amax_v = torch.maximum(amax_v, vv.abs().amax(dim=(0, 2, 3)))
         amax_k = torch.maximum(amax_k, new_key.float().abs().amax(dim=(0, 2)))
         amax_v = torch.maximum(amax_v, new_value.float().abs().amax(dim=(0, 2)))
         k_scale = (amax_k / FP8_MAX).float()
         v_scale = (amax_v / FP8_MAX).float()
-        sg = torch.Generator(device=dev).manual_seed(seed + 2)
-        for i in range(0, pool_blocks, step):
-            m = min(step, pool_blocks - i)
-            kk = torch.randn(m, hkv, bs, d, generator=sg, device=dev)
-            vv = torch.randn(m, hkv, bs, d, generator=sg, device=dev)
+        for i, m, kk, vv in _fp8_source_chunks(pool_shape, dev, seed):
             k_pool[i:i + m] = (kk / k_scale[None, :, None, None]).clamp(-FP8_MAX, FP8_MAX).to(shape.kv_dtype)
             v_pool[i:i + m] = (vv / v_scale[None, :, None, None]).clamp(-FP8_MAX, FP8_MAX).to(shape.kv_dtype)
     else:

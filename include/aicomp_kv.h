@@ -59,7 +59,10 @@ const char* aicomp_kv_last_error(void);
  *   key, value     [T, Hkv, D] of in_dtype; element (t,h,d) is at
  *                  t*kv_token_stride + h*kv_head_stride + d  (strides in elements)
  *   k_pool, v_pool pools of pool_dtype
- *   slot_mapping   [T] int64; slot < 0 skips the row; slots must be distinct
+ *   slot_mapping   [T] int64; slots must be distinct.  A row whose slot is negative (padding)
+ *                  or >= num_blocks * block_size (outside the pool) is skipped without an error:
+ *                  the library cannot report a per-row fault from a kernel, so a planner that
+ *                  wants to hear about such rows checks its slots on the host
  *   in_dtype == pool_dtype                  raw copy, bit-exact
  *   in_dtype f32/bf16, pool_dtype FP8_E4M3  code = e4m3_rne(clamp(x / scale[h], +-448)),
  *                                           k_scale / v_scale [Hkv] float, required
@@ -80,11 +83,21 @@ int aicomp_kv_append(const void* key, const void* value,
  * including the .contiguous() prefix copies it is fed from (kv_cache.py:391-392).
  *
  *   out, query      [B, Hq, D] of q_dtype, contiguous
- *   block_table     [B, max_blocks_per_seq] int32, row stride block_table_stride
- *   context_lens    [B] int32, tokens to attend to (0 -> the output row is zero)
+ *   block_table     [B, max_blocks_per_seq] int32, row stride block_table_stride.  Entries are
+ *                   trusted to lie in [0, num_blocks); one that does not is clamped into the
+ *                   pool (no fault, and no error: the row then attends over another block)
+ *   context_lens    [B] int32, tokens to attend to (0 -> the output row is zero); a length
+ *                   beyond max_blocks_per_seq * block_size is cut to that
  *   scale           softmax scale (the reference's default is 1/sqrt(D))
  *   kv_dtype FP8    k_scale / v_scale [Hkv] float dequantisation factors, fused
- *                   into the loads
+ *                   into the loads.  Accuracy: against attention over the dequantised
+ *                   codes the result meets the bf16 tolerance (1e-2 abs or 2e-2 rel);
+ *                   against attention over the values BEFORE quantisation (unit-variance
+ *                   K and V, absmax scales) the error per output element is at most
+ *                   6e-2 abs or 1e-1 rel for rows attending to >= 1024 keys, and at most
+ *                   1e-2 + min(0.3, 1.6 / sqrt(n)) for a row of n keys (the format's
+ *                   3 mantissa bits; averaging over n keys shrinks it).  The same holds
+ *                   for aicomp_paged_prefill_attn over an fp8 pool.
  *   partition_size  split-K (flash-decoding) tokens per partition; 0 = choose
  *                   from the shape (balanced schedule: every wave gets the same
  *                   number of 32-token tiles); a multiple of block_size otherwise.
@@ -122,6 +135,10 @@ int aicomp_paged_decode_attn(void* out, const void* query,
  *   context_lens        lengths INCLUDING the new token
  * Everything else as aicomp_paged_decode_attn.  The result equals aicomp_kv_append of those
  * rows followed by aicomp_paged_decode_attn: the pool contents are bit-identical.
+ * Row b is stored only if 1 <= context_lens[b] <= max_blocks_per_seq * block_size and its
+ * table entry lies in [0, num_blocks); otherwise the pools are left as they are for that
+ * sequence (whichever kernel does the append), and its output row is computed from the pool
+ * contents under the clamping rules above.
  */
 int aicomp_paged_decode_attn_append(void* out, const void* query,
                                     const void* new_key, const void* new_value,

@@ -174,7 +174,8 @@ def test_decode_errors(device):
 
 def test_fp8_decode_vs_dequantised_oracle(device):
     """fp8 e4m3 KV with per-head scales, group 8: within the bf16 tolerance of the
-    oracle run on the dequantised values; wider stated bound vs unquantised."""
+    oracle run on the dequantised values (the wider, stated bound against the unquantised
+    values is test_gpu_fp8_bound.py's)."""
     w = workloads.make_workload("x", device=device, shape=small("llama3_70b_decode_fp8", batch=4))
     ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping, w.k_scale, w.v_scale)
     want = oracle_decode(w)
@@ -240,6 +241,52 @@ def test_fused_append_edge_positions(device):
     assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
     want = oracle_decode(w, ctx=ctx.cpu().numpy())
     assert_close_attn(to_f64(out), want, BF16_ATOL, BF16_RTOL, "fused edge positions")
+
+
+@pytest.mark.parametrize("name,partition", [("llama3_8b_decode", 0), ("llama3_8b_decode", 256),
+                                            ("llama32_1b_decode", 0), ("llama3_70b_decode_fp8", 0)])
+def test_fused_append_skips_rows_the_table_cannot_place(device, name, partition):
+    """A table entry outside the pool, or a length beyond the table, must not make the fused call store
+    the new row anywhere: the in-kernel append and the separate one-token append (taken when the new
+    rows cannot be read 16 bytes at a time) leave bit-identical pools, untouched for those rows."""
+    w = workloads.make_workload("x", device=device, seed=3, shape=small(name, batch=6))
+    B, nb = 6, w.k_pool.shape[0]
+    width = w.block_table.shape[1]
+    table = w.block_table.clone()
+    ctx = w.context_lens.clone()
+    last = ((ctx - 1) // 16).long()
+    table[1, last[1]] = -1                         # below the pool
+    table[2, last[2]] = nb + 7                     # above the pool
+    ctx[4] = width * 16 + 5                        # longer than the table is wide
+    bits = lambda t: t.view(torch.uint8)
+    pools = []
+    outs = []
+    for aligned in (True, False):
+        k2, v2 = w.k_pool.clone(), w.v_pool.clone()
+        if aligned:
+            nk, nv = w.new_key, w.new_value
+        else:                                      # same values at an address that is not a multiple of 16
+            flat_k = torch.zeros(w.new_key.numel() + 1, dtype=w.new_key.dtype, device=device)
+            flat_v = torch.zeros_like(flat_k)
+            nk, nv = flat_k[1:].view_as(w.new_key), flat_v[1:].view_as(w.new_value)
+            nk.copy_(w.new_key); nv.copy_(w.new_value)
+            assert nk.data_ptr() % 16 != 0
+        out = torch.full_like(w.query, float("nan"))
+        ops.paged_decode_attn(out, w.query, k2, v2, table, ctx, w.scale, k_scale=w.k_scale, v_scale=w.v_scale,
+                              new_key=nk, new_value=nv, partition_size=partition)
+        torch.cuda.synchronize()
+        pools.append((k2, v2)); outs.append(out)
+    (ka, va), (kb, vb) = pools
+    assert torch.equal(bits(ka), bits(kb)) and torch.equal(bits(va), bits(vb)), "fused and unfused pools differ"
+    # rows 0, 3, 5 were stored, and nothing else changed: compare with a slot-mapped append of those rows
+    k3, v3 = w.k_pool.clone(), w.v_pool.clone()
+    slots = w.slot_mapping.clone()
+    slots[[1, 2, 4]] = -1
+    ops.kv_append(w.new_key, w.new_value, k3, v3, slots, w.k_scale, w.v_scale)
+    assert torch.equal(bits(ka), bits(k3)) and torch.equal(bits(va), bits(v3)), "an unplaceable row was stored"
+    good = [0, 3, 5]
+    assert torch.equal(outs[0][good].view(torch.int16), outs[1][good].view(torch.int16))
+    assert torch.isfinite(outs[0][good].float()).all()
 
 
 def test_fp8_all_codes_through_the_decode_kernel(device):

@@ -1,0 +1,105 @@
+"""fp8-e4m3 KV against the UNQUANTISED model: the stated, frozen bound.
+
+The other fp8 tests compare the kernels with the oracle run on the dequantised codes (what the
+kernel should compute from the pool it is given: bf16 tolerance).  What a user of fp8 KV needs
+as well is the distance to the result the same attention gives on the values before they were
+quantised.  That error is a property of the format (3 mantissa bits, per-KV-head absmax scale)
+and of the data, not of the kernel (averaging over n keys shrinks it like 1/sqrt(n)); it is
+measured here on the benchmark's own distribution (K, V ~ N(0, 1) with absmax scales,
+q ~ N(0, 1), scale 1/sqrt(D)) and frozen, per output element, with the float64 oracle on the
+float32 source rows as the unquantised result:
+
+    rows attending to >= 1024 keys (the Llama-3-70B decode shape's contexts):
+        |out_fp8 - out_unq| <= 6e-2   or   <= 1e-1 * |out_unq|
+    any row, n keys:
+        |out_fp8 - out_unq| <= 1e-2 + min(0.3, 1.6 / sqrt(n))
+
+Measured on MI355X: decode at full size 8.4e-3 (sampled sequences, the shortest included);
+prefill rows 0.19 at 1-8 keys, 0.13 at 16, 0.09 at 32-64, 0.07 at 128, 0.06 at 256, 0.03 at 512,
+0.02 at 1024-2048 (six seeds, head_dim 64 and 128): between 1.6 and 3 times inside the rule.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from aicomp_amd import ops, workloads
+from oracle import paged_kv_oracle as orc
+from helpers import assert_close_attn, raw, to_f64
+
+pytestmark = pytest.mark.gpu
+
+# the stated wider bound for fp8 KV vs the unquantised float result (also in include/aicomp_kv.h)
+FP8_ATOL, FP8_RTOL = 6e-2, 1e-1                 # rows with >= 1024 keys
+
+
+def fp8_atol_for_keys(n):
+    return 1e-2 + np.minimum(0.3, 1.6 / np.sqrt(n))
+
+
+def test_fp8_decode_vs_unquantised_model_full_size(device):
+    """Llama-3-70B per-GPU decode shape (batch 128, 64 / 8 heads, contexts 1024..8192) at full size:
+    fused append + decode over the fp8 pools, sampled sequences against float64 attention over the
+    float32 rows the pools were quantised from."""
+    w = workloads.make_workload("llama3_70b_decode_fp8", device=device)
+    out = torch.full_like(w.query, float("nan"))
+    ops.paged_decode_attn(out, w.query, w.k_pool, w.v_pool, w.block_table, w.context_lens, w.scale,
+                          w.k_scale, w.v_scale, new_key=w.new_key, new_value=w.new_value)
+    torch.cuda.synchronize()
+    order = sorted(range(w.num_seqs), key=lambda i: w.ctx_list[i])
+    sample = [order[0], order[len(order) // 2], order[-1], 5]
+    src = workloads.unquantised_context(w, sample)
+    worst = 0.0
+    for s, (k, v) in zip(sample, src):
+        q = orc.decode_elements(raw(w.query[s:s + 1]), "bf16")
+        want = orc.attend_contiguous(q, k.double().cpu().numpy(), v.double().cpu().numpy(), w.scale)[0]
+        got = to_f64(out[s])
+        worst = max(worst, float(np.abs(got - want).max()))
+        assert_close_attn(got, want, FP8_ATOL, FP8_RTOL, f"fp8 decode vs unquantised, sequence {s}")
+    print(f"fp8 decode vs unquantised: max abs error {worst:.3e} over sequences {sample}")
+
+
+@pytest.mark.parametrize("d,hq,hkv", [(128, 16, 2), (64, 8, 2)])
+def test_fp8_prefill_vs_unquantised_model(device, d, hq, hkv):
+    """Chunks (fresh prompts and continuations) over fp8 pools against float64 causal attention over
+    the float32 K/V the pools were quantised from."""
+    g = torch.Generator().manual_seed(21)
+    priors, news, bs = [0, 700, 64, 0, 1500], [300, 130, 512, 40, 64], 16
+    ctx = [p + n for p, n in zip(priors, news)]
+    need = [math.ceil(c / bs) for c in ctx]
+    nb = sum(need) + 3
+    perm = torch.randperm(nb, generator=g)
+    table = torch.zeros(len(ctx), max(need), dtype=torch.int32)
+    cur = 0
+    for s, k in enumerate(need):
+        table[s, :k] = perm[cur:cur + k].to(torch.int32)
+        cur += k
+    kf = torch.randn(nb, hkv, bs, d, generator=g)
+    vf = torch.randn(nb, hkv, bs, d, generator=g)
+    ks = (kf.abs().amax(dim=(0, 2, 3)) / 448).float()
+    vs = (vf.abs().amax(dim=(0, 2, 3)) / 448).float()
+    k_pool = (kf / ks[None, :, None, None]).to(torch.float8_e4m3fn).to(device)
+    v_pool = (vf / vs[None, :, None, None]).to(torch.float8_e4m3fn).to(device)
+    T = sum(news)
+    q = torch.randn(T, hq, d, generator=g).to(torch.bfloat16)
+    cu = torch.tensor([0] + list(np.cumsum(news)), dtype=torch.int32)
+    out = torch.full((T, hq, d), float("nan"), dtype=torch.bfloat16, device=device)
+    ops.paged_prefill_attn(out, q.to(device), k_pool, v_pool, table.to(device),
+                           torch.tensor(ctx, dtype=torch.int32, device=device), cu.to(device),
+                           1 / math.sqrt(d), max_q_len=max(news), k_scale=ks.to(device), v_scale=vs.to(device))
+    torch.cuda.synchronize()
+    want = orc.paged_prefill_attn(raw(q), kf.numpy(), vf.numpy(), table.numpy(), ctx, cu.numpy(),
+                                  1 / math.sqrt(d), "bf16", "f32")
+    got = to_f64(out)
+    err = np.abs(got - want)
+    # keys seen by every query row: prior + position in the chunk + 1
+    nkeys = np.concatenate([p + 1 + np.arange(n) for p, n in zip(priors, news)])
+    print(f"fp8 prefill vs unquantised (D {d}): max abs error {err.max():.3e}, "
+          f"{err[nkeys >= 512].max():.3e} on rows with >= 512 keys")
+    assert np.isfinite(got).all()
+    over = err > fp8_atol_for_keys(nkeys)[:, None, None]
+    assert not over.any(), f"{over.sum()} elements beyond the stated fp8 bound, worst {err[over].max():.3e}"
+    long_rows = nkeys >= 1024
+    assert long_rows.any()
+    assert_close_attn(got[long_rows], want[long_rows], FP8_ATOL, FP8_RTOL, f"fp8 prefill rows with >= 1024 keys, D {d}")
