@@ -26,7 +26,7 @@ SYMBOLS = (
     "aicomp_sample_tokens",
 )
 
-F32, BF16, FP8_E4M3 = 0, 1, 2
+F32, BF16, FP8_E4M3, F16 = 0, 1, 2, 3
 
 _lock = threading.Lock()
 _lib = None

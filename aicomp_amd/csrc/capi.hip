@@ -110,8 +110,8 @@ int aicomp_rope_kv_append(const void* q_in, void* q_out, int64_t q_token_stride,
                    "rope_kv_append: bad sizes (Hq %d, Hkv %d, D %d, BS %d, blocks %lld, table rows %lld)",
                    num_q_heads, num_kv_heads, head_dim, block_size, (long long)num_blocks,
                    (long long)table_rows);
-    AICOMP_REQUIRE(in_dtype == AICOMP_KV_F32 || in_dtype == AICOMP_KV_BF16, AICOMP_KV_EUNSUPPORTED,
-                   "rope_kv_append: inputs must be float32 or bfloat16 (got %d)", in_dtype);
+    AICOMP_REQUIRE(in_dtype == AICOMP_KV_F32 || is_16bit_float(in_dtype), AICOMP_KV_EUNSUPPORTED,
+                   "rope_kv_append: inputs must be float32, bfloat16 or float16 (got %d)", in_dtype);
     AICOMP_REQUIRE(pool_dtype == in_dtype || pool_dtype == AICOMP_KV_FP8_E4M3, AICOMP_KV_EUNSUPPORTED,
                    "rope_kv_append: pool type %d must be the input type %d or fp8-e4m3", pool_dtype,
                    in_dtype);
@@ -146,8 +146,8 @@ int aicomp_sample_tokens(int64_t* out, const void* logits, int64_t row_stride, f
     AICOMP_REQUIRE(out && logits, AICOMP_KV_EINVAL, "sample_tokens: null pointer");
     AICOMP_REQUIRE(vocab > 0 && row_stride >= vocab, AICOMP_KV_EINVAL,
                    "sample_tokens: bad sizes (vocab %d, row stride %lld)", vocab, (long long)row_stride);
-    AICOMP_REQUIRE(logits_dtype == AICOMP_KV_F32 || logits_dtype == AICOMP_KV_BF16, AICOMP_KV_EUNSUPPORTED,
-                   "sample_tokens: logits must be float32 or bfloat16 (got %d)", logits_dtype);
+    AICOMP_REQUIRE(logits_dtype == AICOMP_KV_F32 || is_16bit_float(logits_dtype), AICOMP_KV_EUNSUPPORTED,
+                   "sample_tokens: logits must be float32, bfloat16 or float16 (got %d)", logits_dtype);
     if (!greedy) {
         AICOMP_REQUIRE(uniforms, AICOMP_KV_EINVAL, "sample_tokens: sampling needs uniforms");
         AICOMP_REQUIRE(temperature > 0.f, AICOMP_KV_EINVAL,
@@ -174,8 +174,8 @@ static int resolve_parts(int64_t rows, int hkv, int bs, int max_blocks, int& par
 }
 
 static bool streamk_shape(int batch, int hq, int hkv, int d, int bs, int q_dtype, int kv_dtype) {
-    return d == 128 && bs == 16 && q_dtype == AICOMP_KV_BF16 &&
-           (kv_dtype == AICOMP_KV_BF16 || kv_dtype == AICOMP_KV_FP8_E4M3) && hq / hkv <= 16 &&
+    return d == 128 && bs == 16 && is_16bit_float(q_dtype) &&
+           (kv_dtype == q_dtype || kv_dtype == AICOMP_KV_FP8_E4M3) && hq / hkv <= 16 &&
            batch <= 1024;
 }
 
@@ -235,7 +235,7 @@ static int decode_impl(void* out, const void* query, const void* new_key, const 
     a.num_parts = resolve_parts(batch, num_kv_heads, block_size, max_blocks_per_seq, a.partition_size);
     a.stream = (hipStream_t)stream;
     // the matrix-core kernels append the new rows themselves when they can read them 16 bytes at a time
-    const bool injectable = fused && q_dtype == AICOMP_KV_BF16 && kv_token_stride % 8 == 0 &&
+    const bool injectable = fused && is_16bit_float(q_dtype) && kv_token_stride % 8 == 0 &&
                             kv_head_stride % 8 == 0 && (uintptr_t)new_key % 16 == 0 &&
                             (uintptr_t)new_value % 16 == 0;
     if (partition_size == 0 && decode_streamk_supported(a)) {

@@ -34,6 +34,7 @@ inline int dtype_size(int dt) {
     switch (dt) {
         case AICOMP_KV_F32: return 4;
         case AICOMP_KV_BF16: return 2;
+        case AICOMP_KV_F16: return 2;
         case AICOMP_KV_FP8_E4M3: return 1;
         default: return 0;
     }
@@ -41,7 +42,10 @@ inline int dtype_size(int dt) {
 
 // --------------------------------------------------------- element types ---
 struct bf16_t { uint16_t bits; };
+struct f16_t { uint16_t bits; };
 struct fp8_t { uint8_t bits; };
+
+inline bool is_16bit_float(int dt) { return dt == AICOMP_KV_BF16 || dt == AICOMP_KV_F16; }
 
 constexpr int WAVE = 64;
 constexpr float LOG2E = 1.4426950408889634f;
@@ -56,6 +60,14 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
     if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
     u += 0x7fffu + ((u >> 16) & 1u);
     return (uint16_t)(u >> 16);
+}
+
+// IEEE binary16 <-> float (hardware conversions, round to nearest even; what torch's cast does)
+__device__ __forceinline__ float f16_to_f32(uint16_t b) {
+    return (float)__builtin_bit_cast(_Float16, b);
+}
+__device__ __forceinline__ uint16_t f32_to_f16(float f) {
+    return __builtin_bit_cast(uint16_t, (_Float16)f);
 }
 
 // OCP e4m3 code -> float: gfx950's hardware conversion (byte 0 of the word)
@@ -84,6 +96,17 @@ template <> struct Vec16<bf16_t> {
         }
     }
 };
+template <> struct Vec16<f16_t> {
+    static constexpr int N = 8;
+    __device__ __forceinline__ static void unpack(const uint4& r, float* f) {
+        const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = f16_to_f32((uint16_t)(w[i] & 0xffffu));
+            f[2 * i + 1] = f16_to_f32((uint16_t)(w[i] >> 16));
+        }
+    }
+};
 template <> struct Vec16<fp8_t> {
     static constexpr int N = 16;
     __device__ __forceinline__ static void unpack(const uint4& r, float* f) {
@@ -101,10 +124,82 @@ template <> struct Vec16<fp8_t> {
 template <typename T> __device__ __forceinline__ float load_elem(const T* p);
 template <> __device__ __forceinline__ float load_elem<float>(const float* p) { return *p; }
 template <> __device__ __forceinline__ float load_elem<bf16_t>(const bf16_t* p) { return bf16_to_f32(p->bits); }
+template <> __device__ __forceinline__ float load_elem<f16_t>(const f16_t* p) { return f16_to_f32(p->bits); }
 
 template <typename T> __device__ __forceinline__ void store_elem(T* p, float v);
 template <> __device__ __forceinline__ void store_elem<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void store_elem<bf16_t>(bf16_t* p, float v) { p->bits = f32_to_bf16(v); }
+template <> __device__ __forceinline__ void store_elem<f16_t>(f16_t* p, float v) { p->bits = f32_to_f16(v); }
+
+// ------------------------------------- 16-bit formats of the matrix-core kernels ---
+// The decode and prefill kernels are written once over a 16-bit element format: operands travel
+// as raw 128-bit words, and everything that depends on the format (the MFMA instruction, the
+// float <-> element conversions, fp8 widening, the pair sum) goes through one of these.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+struct Bf16Fmt {
+    typedef bf16_t elem;
+    static constexpr int DT = AICOMP_KV_BF16;
+    // D[16x16] += A[16x32] * B[32x16]: v_mfma_f32_16x16x32_bf16
+    __device__ __forceinline__ static f32x4_t mfma(const uint4& a, const uint4& b, const f32x4_t& c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                       __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+    // two floats -> two packed elements, round to nearest even (v_cvt_pk_bf16_f32)
+    __device__ __forceinline__ static uint32_t pack(float lo, float hi) {
+        const bf16x2_t p = {(__bf16)lo, (__bf16)hi};
+        return __builtin_bit_cast(uint32_t, p);
+    }
+    __device__ __forceinline__ static float to_f32(uint16_t b) { return bf16_to_f32(b); }
+    __device__ __forceinline__ static uint16_t from_f32(float f) { return f32_to_bf16(f); }
+    // 8 e4m3 codes -> 8 elements, exact (3 mantissa bits); the scale operand is 1.0
+    __device__ __forceinline__ static uint4 from_fp8(const uint2& r) {
+        uint4 o;
+        o.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.x, 1.0f, false));
+        o.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.x, 1.0f, true));
+        o.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.y, 1.0f, false));
+        o.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.y, 1.0f, true));
+        return o;
+    }
+    // acc + lo + hi of a packed pair (v_dot2c_f32_bf16 against a pair of ones)
+    __device__ __forceinline__ static float pair_sum(uint32_t pp, float acc) {
+        const bf16x2_t one = {(__bf16)1.0f, (__bf16)1.0f};
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pp), one, acc, false);
+    }
+    static constexpr uint32_t SIGN_PAIR = 0x80008000u;
+};
+
+struct F16Fmt {
+    typedef f16_t elem;
+    static constexpr int DT = AICOMP_KV_F16;
+    __device__ __forceinline__ static f32x4_t mfma(const uint4& a, const uint4& b, const f32x4_t& c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
+                                                      __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    }
+    __device__ __forceinline__ static uint32_t pack(float lo, float hi) {       // v_cvt_pk_f16_f32
+        const f16x2_t p = {(_Float16)lo, (_Float16)hi};
+        return __builtin_bit_cast(uint32_t, p);
+    }
+    __device__ __forceinline__ static float to_f32(uint16_t b) { return f16_to_f32(b); }
+    __device__ __forceinline__ static uint16_t from_f32(float f) { return f32_to_f16(f); }
+    __device__ __forceinline__ static uint4 from_fp8(const uint2& r) {
+        uint4 o;
+        o.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(r.x, 1.0f, false));
+        o.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(r.x, 1.0f, true));
+        o.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(r.y, 1.0f, false));
+        o.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(r.y, 1.0f, true));
+        return o;
+    }
+    __device__ __forceinline__ static float pair_sum(uint32_t pp, float acc) {  // v_dot2c_f32_f16
+        const f16x2_t one = {(_Float16)1.0f, (_Float16)1.0f};
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, pp), one, acc, false);
+    }
+    static constexpr uint32_t SIGN_PAIR = 0x80008000u;
+};
 
 // ------------------------------------------------- split-K workspace view ---
 // part_acc [rows][Hq][P][D] float : sum_j 2^(s_j - m) v_j   (not normalised)

@@ -45,6 +45,12 @@ template <> struct KvLoad<bf16_t> {
     __device__ __forceinline__ static Raw raw(const bf16_t* p) { return stream_ld16(p); }
     __device__ __forceinline__ static void unpack(const Raw& r, float* f) { Vec16<bf16_t>::unpack(r, f); }
 };
+template <> struct KvLoad<f16_t> {
+    static constexpr int N = 8;
+    typedef uint4 Raw;
+    __device__ __forceinline__ static Raw raw(const f16_t* p) { return stream_ld16(p); }
+    __device__ __forceinline__ static void unpack(const Raw& r, float* f) { Vec16<f16_t>::unpack(r, f); }
+};
 template <> struct KvLoad<fp8_t> {
     static constexpr int N = 8;
     typedef uint2 Raw;
@@ -342,6 +348,10 @@ int launch_split_reduce(const DecodeArgs& a) {
         hipLaunchKernelGGL(split_reduce_kernel<float>, grid, dim3(threads), 0, a.stream,
                            (float*)a.out, a.ws.acc, a.ws.ml, a.context_lens, a.cu_q_lens,
                            a.num_seqs, a.hq, group, a.d, a.partition_size, a.num_parts, a.v_scale);
+    else if (a.q_dtype == AICOMP_KV_F16)
+        hipLaunchKernelGGL(split_reduce_kernel<f16_t>, grid, dim3(threads), 0, a.stream,
+                           (f16_t*)a.out, a.ws.acc, a.ws.ml, a.context_lens, a.cu_q_lens,
+                           a.num_seqs, a.hq, group, a.d, a.partition_size, a.num_parts, a.v_scale);
     else
         hipLaunchKernelGGL(split_reduce_kernel<bf16_t>, grid, dim3(threads), 0, a.stream,
                            (bf16_t*)a.out, a.ws.acc, a.ws.ml, a.context_lens, a.cu_q_lens,
@@ -399,9 +409,13 @@ int launch_decode_generic(const DecodeArgs& a) {
         rc = launch_generic_t<bf16_t, bf16_t>(a, p);
     else if (a.kv_dtype == AICOMP_KV_FP8_E4M3 && a.q_dtype == AICOMP_KV_BF16)
         rc = launch_generic_t<fp8_t, bf16_t>(a, p);
+    else if (a.kv_dtype == AICOMP_KV_F16 && a.q_dtype == AICOMP_KV_F16)
+        rc = launch_generic_t<f16_t, f16_t>(a, p);
+    else if (a.kv_dtype == AICOMP_KV_FP8_E4M3 && a.q_dtype == AICOMP_KV_F16)
+        rc = launch_generic_t<fp8_t, f16_t>(a, p);
     else {
         set_error("paged attention: unsupported type pair (query %d, pool %d); supported: "
-                  "f32/f32, bf16/bf16, bf16/fp8", a.q_dtype, a.kv_dtype);
+                  "f32/f32, bf16/bf16, f16/f16, bf16/fp8, f16/fp8", a.q_dtype, a.kv_dtype);
         return AICOMP_KV_EUNSUPPORTED;
     }
     if (rc != AICOMP_KV_OK) return rc;

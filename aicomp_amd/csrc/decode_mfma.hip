@@ -5,8 +5,8 @@
 // and the two .contiguous() prefix copies that feed it (kv_cache.py:391-392):
 // K and V are read once, in place, through the block table.
 //
-// Shape covered: head_dim 128, block_size 16, bf16 queries, bf16 or fp8-e4m3
-// pools, up to 16 query heads per KV head; and head_dim 64 (up to 8 heads per KV
+// Shape covered: head_dim 128, block_size 16, bf16 or fp16 queries, pools of the query type or
+// fp8-e4m3 (the kernels are written over a 16-bit element format, see common.h), up to 16 query heads per KV head; and head_dim 64 (up to 8 heads per KV
 // head) by treating two consecutive tokens, which are contiguous in the pool, as
 // one 128-element row: every head takes two B-operand columns, one per token
 // parity, with the query in the matching half of the row and zeros in the other,
@@ -26,7 +26,7 @@
 //              block, wave-uniform (scalar).
 // K            staged through a wave-private LDS tile (row stride 272 B, so the
 //              16 rows a quarter-wave reads hit distinct banks) and read back
-//              as the A operand of  S^T = K Q^T  (v_mfma_f32_16x16x32_bf16),
+//              as the A operand of  S^T = K Q^T  (v_mfma_f32_16x16x32_bf16 / _f16),
 //              the G query heads (padded to 16 columns) sharing every K tile.
 // V            never touches LDS.  Lane (c = l%16, q = l/16) of load i holds
 //              dims 8c..8c+7 of token 4i+q; picking the j-th 16-bit half of
@@ -44,10 +44,6 @@
 #include <atomic>
 
 namespace aicomp {
-
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 namespace {
 
@@ -77,27 +73,10 @@ struct MfmaParams {
     float* ws_acc;
     float* ws_ml;
     // fused append (optional): row b of new_key / new_value is token context_lens[b]-1
-    const bf16_t* new_key;
-    const bf16_t* new_value;
+    const uint16_t* new_key;
+    const uint16_t* new_value;
     int64_t new_token_stride, new_head_stride;     // elements
 };
-
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-    bf16x2_t p = {(__bf16)lo, (__bf16)hi};
-    return __builtin_bit_cast(uint32_t, p);
-}
-
-// 8 fp8 codes -> 8 bf16
-__device__ __forceinline__ uint4 fp8x8_to_bf16x8(uint2 r) {
-    // gfx950 converts two e4m3 codes straight to two packed bf16 (exact: 3 mantissa bits);
-    // the scale operand is 1.0
-    uint4 o;
-    o.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.x, 1.0f, false));
-    o.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.x, 1.0f, true));
-    o.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.y, 1.0f, false));
-    o.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.y, 1.0f, true));
-    return o;
-}
 
 template <bool FP8> struct TileRegs;
 template <> struct TileRegs<false> { uint4 r[8]; };
@@ -165,9 +144,10 @@ __device__ __forceinline__ void load_tile_pair(TileRegs<FP8>& t, const void* poo
     }
 }
 
-template <bool FP8>
-__device__ __forceinline__ uint4 tile_bf16(const TileRegs<FP8>& t, int i) {
-    if constexpr (FP8) return fp8x8_to_bf16x8(t.r[i]);
+// load i of a tile as eight elements of the query's 16-bit format E (fp8 pools are widened, exactly)
+template <typename E, bool FP8>
+__device__ __forceinline__ uint4 tile_elems(const TileRegs<FP8>& t, int i) {
+    if constexpr (FP8) return E::from_fp8(t.r[i]);
     else return t.r[i];
 }
 
@@ -186,9 +166,9 @@ struct WaveState {
 // MASK: the tile crosses `end`; scores beyond it are dropped and their V rows zeroed.
 // PAIR: rows are token pairs (head_dim 64): row r of the tile holds tokens tile_start + 2r and
 // + 2r + 1, the B-operand columns are (head, parity) pairs, column c scoring token 2r + (c & 1).
-template <bool FP8, bool NEXT, bool MASK, bool PAIR = false>
+template <typename E, bool FP8, bool NEXT, bool MASK, bool PAIR = false>
 __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, TileRegs<FP8>& vr,
-                                             const bf16x8_t (&qf)[4], unsigned char* kt, int wr_off,
+                                             const uint4 (&qf)[4], unsigned char* kt, int wr_off,
                                              int rd_off, const void* k_pool, const void* v_pool,
                                              int64_t nb0, int64_t nb1, int hkv, int kvh_next, int lane,
                                              int g4, int tile_start, int end, float cmul,
@@ -196,7 +176,7 @@ __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, T
     // ---- K tile -> LDS, then prefetch the next K tile into the same registers
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        uint4 kk = tile_bf16<FP8>(kr, i);
+        uint4 kk = tile_elems<E, FP8>(kr, i);
         // PAIR: a row's two tokens share every dot product (the query column is zero over the other
         // token's half), so a token beyond the context must not leave non-finite values in the row
         if (PAIR && MASK && tile_start + 2 * (4 * i + g4) + ((lane & 15) >> 3) >= end) kk = make_uint4(0, 0, 0, 0);
@@ -213,8 +193,8 @@ __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, T
     for (int s = 0; s < 4; ++s) {
         const uint4 a0 = *(const uint4*)(kt + rd_off + s * 64);
         const uint4 a1 = *(const uint4*)(kt + rd_off + 16 * KROW + s * 64);
-        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a0), qf[s], s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a1), qf[s], s1, 0, 0, 0);
+        s0 = E::mfma(a0, qf[s], s0);
+        s1 = E::mfma(a1, qf[s], s1);
     }
     // lane (head r16, g4) now holds tokens tile_start + 16a + 4i + g4 in s_a[i]
     float sc[8];
@@ -249,15 +229,14 @@ __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, T
     }
     // P^T as the B operand: k-slot 4a + i <-> token 16a + 4i + g4, this lane's own values
     uint4 pw;
-    pw.x = pack_bf16(pr[0], pr[1]); pw.y = pack_bf16(pr[2], pr[3]);
-    pw.z = pack_bf16(pr[4], pr[5]); pw.w = pack_bf16(pr[6], pr[7]);
-    const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pw);
+    pw.x = E::pack(pr[0], pr[1]); pw.y = E::pack(pr[2], pr[3]);
+    pw.z = E::pack(pr[4], pr[5]); pw.w = E::pack(pr[6], pr[7]);
 
     // ---- V: registers -> A operand of O^T += V^T P^T.  Load i of lane (c, q) is token 4i + q.
     uint4 vv[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        vv[i] = tile_bf16<FP8>(vr, i);
+        vv[i] = tile_elems<E, FP8>(vr, i);
         // PAIR: chunks 8..15 of a row belong to the pair's second token
         const int vtok = PAIR ? tile_start + 2 * (4 * i + g4) + ((lane & 15) >> 3) : tile_start + 4 * i + g4;
         if (MASK && vtok >= end) vv[i] = make_uint4(0, 0, 0, 0);
@@ -278,17 +257,18 @@ __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, T
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j)
-        st.O[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, af[j]), pf, st.O[j], 0, 0, 0);
+        st.O[j] = E::mfma(af[j], pw, st.O[j]);
 }
 
-// 8 floats -> 8 e4m3 codes: clamp(x / scale, +-448), round to nearest even
-__device__ __forceinline__ uint2 quant8_fp8(const uint4& bf, float scale) {
-    const uint32_t w[4] = {bf.x, bf.y, bf.z, bf.w};
+// 8 elements of format E -> 8 e4m3 codes: clamp(x / scale, +-448), round to nearest even
+template <typename E>
+__device__ __forceinline__ uint2 quant8_fp8(const uint4& x, float scale) {
+    const uint32_t w[4] = {x.x, x.y, x.z, x.w};
     float f[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        f[2 * i] = fminf(fmaxf(__uint_as_float(w[i] << 16) / scale, -448.f), 448.f);
-        f[2 * i + 1] = fminf(fmaxf(__uint_as_float(w[i] & 0xffff0000u) / scale, -448.f), 448.f);
+        f[2 * i] = fminf(fmaxf(E::to_f32((uint16_t)(w[i] & 0xffffu)) / scale, -448.f), 448.f);
+        f[2 * i + 1] = fminf(fmaxf(E::to_f32((uint16_t)(w[i] >> 16)) / scale, -448.f), 448.f);
     }
     int lo = 0, hi = 0;
     lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], lo, false);
@@ -302,7 +282,7 @@ __device__ __forceinline__ uint2 quant8_fp8(const uint4& bf, float scale) {
 // (context_lens - 1) takes its K/V row from new_key / new_value instead of what was loaded from
 // the pool, and writes it to the pool (the append itself).  No other wave of the launch reads
 // that token.  A tile row is one token (16 lanes of 8 elements), or with PAIR half a row (8 lanes).
-template <bool FP8, bool PAIR>
+template <typename E, bool FP8, bool PAIR>
 __device__ __forceinline__ void inject_new_row_grid(TileRegs<FP8>& kr, TileRegs<FP8>& vr, const MfmaParams& p,
                                                     int seq, int kvh, int lane, int tile_start, int len,
                                                     const int64_t (&bb)[4]) {
@@ -320,8 +300,8 @@ __device__ __forceinline__ void inject_new_row_grid(TileRegs<FP8>& kr, TileRegs<
     const int64_t blk = bb[blk_i];
     const int64_t dst = ((blk * p.hkv + kvh) * BS + tb) * (DQ / 8) + c;        // 8-element chunks
     if constexpr (FP8) {
-        const uint2 ck = quant8_fp8(nk, p.k_scale[kvh]);
-        const uint2 cv = quant8_fp8(nv, p.v_scale[kvh]);
+        const uint2 ck = quant8_fp8<E>(nk, p.k_scale[kvh]);
+        const uint2 cv = quant8_fp8<E>(nv, p.v_scale[kvh]);
 #pragma unroll
         for (int i = 0; i < 8; ++i)
             if (mine && i == slot) { kr.r[i] = ck; vr.r[i] = cv; }
@@ -334,7 +314,7 @@ __device__ __forceinline__ void inject_new_row_grid(TileRegs<FP8>& kr, TileRegs<
     }
 }
 
-template <bool FP8, bool PAIR>
+template <typename E, bool FP8, bool PAIR>
 __global__ void __launch_bounds__(256, 2)
 paged_decode_mfma_kernel(MfmaParams p) {
     // KV head fastest: the workgroups launched together read the Hkv slices of the same
@@ -366,10 +346,10 @@ paged_decode_mfma_kernel(MfmaParams p) {
     // Q as the B operand of S^T = K Q^T: column = head r16, k-slots = dims 32s + 8*g4 ..
     // PAIR: column c is (head c/2, parity c%2); a row of the K tile is [token 2r | token 2r+1], so
     // the column carries the query in elements 0..63 (parity 0) or 64..127 (parity 1), zeros elsewhere.
-    bf16x8_t qf[4];
+    uint4 qf[4];
     {
         const int h = PAIR ? (r16 >> 1) : r16;
-        const bf16_t* qrow = (const bf16_t*)p.query + ((int64_t)seq * p.hq + kvh * G + min(h, G - 1)) * DQ;
+        const uint16_t* qrow = (const uint16_t*)p.query + ((int64_t)seq * p.hq + kvh * G + min(h, G - 1)) * DQ;
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             const int e0 = 32 * s + 8 * g4;                       // first element of this k-slot in the row
@@ -381,15 +361,15 @@ paged_decode_mfma_kernel(MfmaParams p) {
             }
             uint4 v = *(const uint4*)(qrow + src);
             if (!use) v = make_uint4(0, 0, 0, 0);
-            qf[s] = __builtin_bit_cast(bf16x8_t, v);
+            qf[s] = v;
         }
     }
 
     const int len = min(p.context_lens[seq], p.max_blocks * BS);   // never read past the table row
     if (start >= len) {
         if (len <= 0 && part == 0) {   // nothing to attend to: the output row is defined as zero
-            bf16_t* o = (bf16_t*)p.out + ((int64_t)seq * p.hq + kvh * G) * DQ;
-            for (int i = tid; i < G * DQ; i += blockDim.x) o[i].bits = 0;
+            uint16_t* o = (uint16_t*)p.out + ((int64_t)seq * p.hq + kvh * G) * DQ;
+            for (int i = tid; i < G * DQ; i += blockDim.x) o[i] = 0;
         }
         return;
     }
@@ -443,7 +423,7 @@ paged_decode_mfma_kernel(MfmaParams p) {
         int tt = w;
         for (; tt + NWAVES < ntiles; tt += NWAVES) {      // steady state: never the partition's last tile
             tile_blocks(tt + NWAVES);
-            process_tile<FP8, true, false, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, bb[0],
+            process_tile<E, FP8, true, false, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, bb[0],
                                                  bb[1], p.hkv, kvh, lane, g4, start + tt * TT, end, cmul,
                                                  bb[2], bb[3]);
         }
@@ -456,13 +436,13 @@ paged_decode_mfma_kernel(MfmaParams p) {
             // (and attends over what the clamped table entry holds, like the unfused sequence of calls).
             const int raw_blk = __builtin_amdgcn_readlane(tab, BPT * tt + ((len - 1 - tile_start) >> 4) - tab_first);
             if (p.context_lens[seq] == len && raw_blk >= 0 && raw_blk < p.num_blocks)
-                inject_new_row_grid<FP8, PAIR>(kr, vr, p, seq, kvh, lane, tile_start, len, bb);
+                inject_new_row_grid<E, FP8, PAIR>(kr, vr, p, seq, kvh, lane, tile_start, len, bb);
         }
         if (tile_start + TT > end)
-            process_tile<FP8, false, true, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
+            process_tile<E, FP8, false, true, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
                                                  p.hkv, kvh, lane, g4, tile_start, end, cmul);
         else
-            process_tile<FP8, false, false, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
+            process_tile<E, FP8, false, false, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
                                                   p.hkv, kvh, lane, g4, tile_start, end, cmul);
     }
     const float m = st.m;
@@ -511,8 +491,8 @@ paged_decode_mfma_kernel(MfmaParams p) {
         }
         const int head = kvh * G + h;
         if (direct) {
-            ((bf16_t*)p.out)[((int64_t)seq * p.hq + head) * DQ + dd].bits =
-                f32_to_bf16(den > 0.f ? vs * num / den : 0.f);
+            ((uint16_t*)p.out)[((int64_t)seq * p.hq + head) * DQ + dd] =
+                E::from_f32(den > 0.f ? vs * num / den : 0.f);
         } else {
             const int64_t slot = ((int64_t)seq * p.hq + head) * p.num_parts + part;
             p.ws_acc[slot * DQ + dd] = num;
@@ -559,8 +539,8 @@ struct StreamKParams {
     float* ws_ml;       // [slots][G][2]
     int* ws_rows;       // [rows][2]: first and last part (wave of the row's head) holding a partial of the row
     // fused append (optional): row b of new_key / new_value is token context_lens[b]-1
-    const bf16_t* new_key;
-    const bf16_t* new_value;
+    const uint16_t* new_key;
+    const uint16_t* new_value;
     int64_t new_token_stride, new_head_stride;     // elements
 };
 
@@ -568,7 +548,7 @@ struct StreamKParams {
 // the pool yet.  The 16 lanes that own that row take it from new_key / new_value instead of
 // what they loaded, and write it to the pool (the append itself).  No other wave of this
 // launch reads that token, so no cross-wave ordering is needed.
-template <bool FP8>
+template <typename E, bool FP8>
 __device__ __forceinline__ void inject_new_row(TileRegs<FP8>& kr, TileRegs<FP8>& vr,
                                                const StreamKParams& p, int seq, int kvh, int lane,
                                                int tile_start, int len, int64_t b0, int64_t b1) {
@@ -581,8 +561,8 @@ __device__ __forceinline__ void inject_new_row(TileRegs<FP8>& kr, TileRegs<FP8>&
     const int64_t blk = tau < 16 ? b0 : b1;
     const int64_t dst = ((blk * p.hkv + kvh) * BS + (tau & 15)) * (D / 8) + c;   // 8-element chunks
     if constexpr (FP8) {
-        const uint2 ck = quant8_fp8(nk, p.k_scale[kvh]);
-        const uint2 cv = quant8_fp8(nv, p.v_scale[kvh]);
+        const uint2 ck = quant8_fp8<E>(nk, p.k_scale[kvh]);
+        const uint2 cv = quant8_fp8<E>(nv, p.v_scale[kvh]);
 #pragma unroll
         for (int i = 0; i < 8; ++i)
             if (mine && i == (tau >> 2)) { kr.r[i] = ck; vr.r[i] = cv; }
@@ -601,7 +581,7 @@ __device__ __forceinline__ int sk_tiles(int len, int max_blocks) {
 }
 
 
-template <bool FP8>
+template <typename E, bool FP8>
 __global__ void __launch_bounds__(256, 1)     // one workgroup per CU: a wave may use the whole register file
 streamk_decode_kernel(StreamKParams p) {
     const int tid = threadIdx.x;
@@ -694,15 +674,14 @@ streamk_decode_kernel(StreamKParams p) {
     // raw query rows of (sequence, KV head); columns beyond the group are zeroed by q_operand
     // only when the rows are used, so that issuing the loads never waits for them
     auto load_q = [&](int sq, int kh, uint4 (&q)[4]) {
-        const uint4* qp = (const uint4*)((const bf16_t*)p.query +
+        const uint4* qp = (const uint4*)((const uint16_t*)p.query +
                                          ((int64_t)sq * p.hq + kh * G + min(r16, G - 1)) * D + 8 * g4);
 #pragma unroll
         for (int s = 0; s < 4; ++s) q[s] = qp[s * 4];
     };
-    auto q_operand = [&](const uint4 (&raw)[4], bf16x8_t (&q)[4]) {
+    auto q_operand = [&](const uint4 (&raw)[4], uint4 (&q)[4]) {
 #pragma unroll
-        for (int s = 0; s < 4; ++s)
-            q[s] = __builtin_bit_cast(bf16x8_t, r16 < G ? raw[s] : make_uint4(0, 0, 0, 0));
+        for (int s = 0; s < 4; ++s) q[s] = r16 < G ? raw[s] : make_uint4(0, 0, 0, 0);
     };
     auto load_tab = [&](int sq, int first_block) {
         const int32_t* table = p.block_table + (int64_t)sq * p.block_table_stride;
@@ -710,7 +689,7 @@ streamk_decode_kernel(StreamKParams p) {
     };
 
     int nt = (int)min((int64_t)(row_tiles - t), g1 - g0);          // tiles of the current segment (>= 1)
-    bf16x8_t qf[4];
+    uint4 qf[4];
     uint4 qraw[4];
     load_q(seq, kvh, qraw);
     int tab = load_tab(seq, 2 * t);
@@ -750,7 +729,7 @@ streamk_decode_kernel(StreamKParams p) {
         }
         const bool has_next = more && nseq < B;
         int tabn = 0;
-        bf16x8_t qn[4];
+        uint4 qn[4];
         if (has_next) {
             load_q(nseq, nkvh, qraw);
             tabn = load_tab(nseq, 0);
@@ -765,7 +744,7 @@ streamk_decode_kernel(StreamKParams p) {
         int k = 0;
         for (; k + 1 < nt; ++k) {
             tile_blocks(k + 1, b0, b1);
-            process_tile<FP8, true, false>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, b0, b1,
+            process_tile<E, FP8, true, false>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, b0, b1,
                                            p.hkv, kvh, lane, g4, (t + k) * TILE, len, cmul);
         }
         const int tile_start = (t + k) * TILE;
@@ -776,7 +755,7 @@ streamk_decode_kernel(StreamKParams p) {
             // (and attends over what the clamped table entry holds, like the unfused sequence of calls).
             const int raw_blk = __builtin_amdgcn_readlane(tab, 2 * k + ((len - 1 - tile_start) >> 4) - tab_first);
             if (p.context_lens[seq] == len && raw_blk >= 0 && raw_blk < p.num_blocks)
-                inject_new_row<FP8>(kr, vr, p, seq, kvh, lane, tile_start, len, b0, b1);
+                inject_new_row<E, FP8>(kr, vr, p, seq, kvh, lane, tile_start, len, b0, b1);
         }
         // The segment's last tile always runs the masked body (a full tile simply masks nothing):
         // one prefetching call site, so the prefetched registers need no merging afterwards.
@@ -788,10 +767,10 @@ streamk_decode_kernel(StreamKParams p) {
             tab_ready = tabn;
             b0 = clamp_block(__builtin_amdgcn_readlane(tab_ready, 0), p.num_blocks);
             b1 = clamp_block(__builtin_amdgcn_readlane(tab_ready, 1), p.num_blocks);
-            process_tile<FP8, true, true>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, b0, b1,
+            process_tile<E, FP8, true, true>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, b0, b1,
                                           p.hkv, nkvh, lane, g4, tile_start, len, cmul);
         } else {
-            process_tile<FP8, false, true>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
+            process_tile<E, FP8, false, true>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
                                            p.hkv, kvh, lane, g4, tile_start, len, cmul);
         }
 
@@ -836,8 +815,9 @@ streamk_decode_kernel(StreamKParams p) {
 // no barrier; with S > 1 (a handful of very long rows, hundreds of partials each) the waves of a
 // head take alternate groups of eight partials and add up through LDS.
 constexpr int RED_WGT = 256;       // weights parked in LDS per wave; rows with more partials recompute the rest
+template <typename E>
 __global__ void __launch_bounds__(1024)
-streamk_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws_acc,
+streamk_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ ws_acc,
                       const float* __restrict__ ws_ml, const int* __restrict__ ws_rows,
                       const int32_t* __restrict__ context_lens, int hq, int hkv, int group,
                       const float* __restrict__ v_scale, int head_slots) {
@@ -849,9 +829,9 @@ streamk_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws_acc
     __shared__ float part[16][D];
     float* wgt = wgt_all[wv];
     const int64_t row = (int64_t)seq * hkv + kvh;
-    bf16_t* o = out + ((int64_t)seq * hq + kvh * group + h) * D;
+    uint16_t* o = out + ((int64_t)seq * hq + kvh * group + h) * D;
     if (context_lens[seq] <= 0) {            // no tiles, no partials: the output row is zero (whole workgroup)
-        if (sub == 0) { o[lane].bits = 0; o[lane + 64].bits = 0; }
+        if (sub == 0) { o[lane] = 0; o[lane + 64] = 0; }
         return;
     }
     const int first = ws_rows[2 * row], last = ws_rows[2 * row + 1];
@@ -899,8 +879,8 @@ streamk_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws_acc
         for (int k = 1; k < S; ++k) { n0 += part[wv + k][lane]; n1 += part[wv + k][lane + 64]; }
     }
     const float inv = den > 0.f ? (v_scale ? v_scale[kvh] : 1.f) / den : 0.f;
-    o[lane].bits = f32_to_bf16(n0 * inv);
-    o[lane + 64].bits = f32_to_bf16(n1 * inv);
+    o[lane] = E::from_f32(n0 * inv);
+    o[lane + 64] = E::from_f32(n1 * inv);
 }
 
 }  // namespace
@@ -911,8 +891,8 @@ bool decode_mfma_supported(const DecodeArgs& a) {
     const int group = a.hkv > 0 ? a.hq / a.hkv : 0;
     const bool shape = (a.d == D && group <= 16 && a.partition_size % TILE == 0) ||
                        (a.d == 64 && group <= 8 && a.partition_size % (2 * TILE) == 0);
-    return a.cu_q_lens == nullptr && shape && a.bs == BS && a.q_dtype == AICOMP_KV_BF16 &&
-           (a.kv_dtype == AICOMP_KV_BF16 || a.kv_dtype == AICOMP_KV_FP8_E4M3) && group >= 1 &&
+    return a.cu_q_lens == nullptr && shape && a.bs == BS && is_16bit_float(a.q_dtype) &&
+           (a.kv_dtype == a.q_dtype || a.kv_dtype == AICOMP_KV_FP8_E4M3) && group >= 1 &&
            a.scale > 0.f && a.rows <= 65535 &&
            a.num_parts <= 65535 && ((uintptr_t)a.query % 16 == 0) && ((uintptr_t)a.k_pool % 16 == 0) &&
            ((uintptr_t)a.v_pool % 16 == 0);
@@ -961,19 +941,25 @@ int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
     p.ws_acc = (float*)workspace;
     p.ws_ml = p.ws_acc + slots * group * D;
     p.ws_rows = (int*)(p.ws_ml + slots * group * 2);
-    p.new_key = (const bf16_t*)a.new_key; p.new_value = (const bf16_t*)a.new_value;
+    p.new_key = (const uint16_t*)a.new_key; p.new_value = (const uint16_t*)a.new_value;
     p.new_token_stride = a.new_token_stride; p.new_head_stride = a.new_head_stride;
-    if (a.kv_dtype == AICOMP_KV_FP8_E4M3)
-        hipLaunchKernelGGL(streamk_decode_kernel<true>, dim3(wgs), dim3(256), 0, a.stream, p);
-    else
-        hipLaunchKernelGGL(streamk_decode_kernel<false>, dim3(wgs), dim3(256), 0, a.stream, p);
+    const bool fp8 = a.kv_dtype == AICOMP_KV_FP8_E4M3, f16 = a.q_dtype == AICOMP_KV_F16;
+    if (f16 && fp8) hipLaunchKernelGGL((streamk_decode_kernel<F16Fmt, true>), dim3(wgs), dim3(256), 0, a.stream, p);
+    else if (f16) hipLaunchKernelGGL((streamk_decode_kernel<F16Fmt, false>), dim3(wgs), dim3(256), 0, a.stream, p);
+    else if (fp8) hipLaunchKernelGGL((streamk_decode_kernel<Bf16Fmt, true>), dim3(wgs), dim3(256), 0, a.stream, p);
+    else hipLaunchKernelGGL((streamk_decode_kernel<Bf16Fmt, false>), dim3(wgs), dim3(256), 0, a.stream, p);
     AICOMP_HIP_LAUNCH_CHECK();
     // waves per head in the merge: one, unless rows are few and long (many partials per row)
     const int64_t per_row = (int64_t)p.waves_per_head / a.rows + 2;
     const int sub = per_row > 8 ? 16 / group : 1;
-    hipLaunchKernelGGL(streamk_reduce_kernel, dim3(a.hkv, (unsigned)a.rows), dim3(64 * group * sub), 0, a.stream,
-                       (bf16_t*)a.out, p.ws_acc, p.ws_ml, p.ws_rows, a.context_lens, a.hq, a.hkv, group,
-                       a.v_scale, p.waves_per_head + (int)a.rows);
+    if (f16)
+        hipLaunchKernelGGL(streamk_reduce_kernel<F16Fmt>, dim3(a.hkv, (unsigned)a.rows), dim3(64 * group * sub), 0,
+                           a.stream, (uint16_t*)a.out, p.ws_acc, p.ws_ml, p.ws_rows, a.context_lens, a.hq, a.hkv,
+                           group, a.v_scale, p.waves_per_head + (int)a.rows);
+    else
+        hipLaunchKernelGGL(streamk_reduce_kernel<Bf16Fmt>, dim3(a.hkv, (unsigned)a.rows), dim3(64 * group * sub), 0,
+                           a.stream, (uint16_t*)a.out, p.ws_acc, p.ws_ml, p.ws_rows, a.context_lens, a.hq, a.hkv,
+                           group, a.v_scale, p.waves_per_head + (int)a.rows);
     AICOMP_HIP_LAUNCH_CHECK();
     return AICOMP_KV_OK;
 }
@@ -989,17 +975,23 @@ int launch_decode_mfma(const DecodeArgs& a) {
     p.k_scale = a.k_scale; p.v_scale = a.v_scale;
     p.partition_size = a.partition_size; p.num_parts = a.num_parts;
     p.ws_acc = a.ws.acc; p.ws_ml = a.ws.ml;
-    p.new_key = (const bf16_t*)a.new_key; p.new_value = (const bf16_t*)a.new_value;
+    p.new_key = (const uint16_t*)a.new_key; p.new_value = (const uint16_t*)a.new_value;
     p.new_token_stride = a.new_token_stride; p.new_head_stride = a.new_head_stride;
     dim3 grid((unsigned)a.hkv, (unsigned)a.num_parts, (unsigned)a.rows);
     const bool fp8 = a.kv_dtype == AICOMP_KV_FP8_E4M3;
-    if (a.d == 64) {
-        if (fp8) hipLaunchKernelGGL((paged_decode_mfma_kernel<true, true>), grid, dim3(256), 0, a.stream, p);
-        else hipLaunchKernelGGL((paged_decode_mfma_kernel<false, true>), grid, dim3(256), 0, a.stream, p);
-    } else {
-        if (fp8) hipLaunchKernelGGL((paged_decode_mfma_kernel<true, false>), grid, dim3(256), 0, a.stream, p);
-        else hipLaunchKernelGGL((paged_decode_mfma_kernel<false, false>), grid, dim3(256), 0, a.stream, p);
-    }
+#define AICOMP_LAUNCH_GRID(E)                                                                                       \
+    do {                                                                                                            \
+        if (a.d == 64) {                                                                                            \
+            if (fp8) hipLaunchKernelGGL((paged_decode_mfma_kernel<E, true, true>), grid, dim3(256), 0, a.stream, p); \
+            else hipLaunchKernelGGL((paged_decode_mfma_kernel<E, false, true>), grid, dim3(256), 0, a.stream, p);   \
+        } else {                                                                                                    \
+            if (fp8) hipLaunchKernelGGL((paged_decode_mfma_kernel<E, true, false>), grid, dim3(256), 0, a.stream, p); \
+            else hipLaunchKernelGGL((paged_decode_mfma_kernel<E, false, false>), grid, dim3(256), 0, a.stream, p);  \
+        }                                                                                                           \
+    } while (0)
+    if (a.q_dtype == AICOMP_KV_F16) AICOMP_LAUNCH_GRID(F16Fmt);
+    else AICOMP_LAUNCH_GRID(Bf16Fmt);
+#undef AICOMP_LAUNCH_GRID
     AICOMP_HIP_LAUNCH_CHECK();
     if (a.num_parts > 1) return launch_split_reduce(a);
     return AICOMP_KV_OK;

@@ -183,14 +183,19 @@ int launch_kv_append_last(const void* key, const void* value, int64_t token_stri
 #undef LAUNCH_LAST
     } else {
         AICOMP_REQUIRE(pool_dtype == AICOMP_KV_FP8_E4M3 &&
-                           (in_dtype == AICOMP_KV_BF16 || in_dtype == AICOMP_KV_F32) && d % 4 == 0,
-                       AICOMP_KV_EUNSUPPORTED, "append: only f32/bf16 -> fp8 conversion is supported");
+                           (is_16bit_float(in_dtype) || in_dtype == AICOMP_KV_F32) && d % 4 == 0,
+                       AICOMP_KV_EUNSUPPORTED, "append: only f32/bf16/f16 -> fp8 conversion is supported");
         AICOMP_REQUIRE(k_scale && v_scale, AICOMP_KV_EINVAL, "append: an fp8 pool needs k_scale and v_scale");
         const int64_t total = (int64_t)batch * hkv * (d / 4);
         const unsigned blocks = (unsigned)((total + threads - 1) / threads);
         if (in_dtype == AICOMP_KV_BF16)
             hipLaunchKernelGGL(kv_append_last_quant<bf16_t>, dim3(blocks), dim3(threads), 0, stream,
                                (const bf16_t*)key, (const bf16_t*)value, token_stride, head_stride,
+                               (uint32_t*)k_pool, (uint32_t*)v_pool, block_table, block_table_stride,
+                               context_lens, k_scale, v_scale, total, hkv, d / 4, bs, max_blocks, num_blocks);
+        else if (in_dtype == AICOMP_KV_F16)
+            hipLaunchKernelGGL(kv_append_last_quant<f16_t>, dim3(blocks), dim3(threads), 0, stream,
+                               (const f16_t*)key, (const f16_t*)value, token_stride, head_stride,
                                (uint32_t*)k_pool, (uint32_t*)v_pool, block_table, block_table_stride,
                                context_lens, k_scale, v_scale, total, hkv, d / 4, bs, max_blocks, num_blocks);
         else
@@ -241,9 +246,9 @@ int launch_kv_append(const void* key, const void* value, int64_t token_stride, i
         }
     } else {
         AICOMP_REQUIRE(pool_dtype == AICOMP_KV_FP8_E4M3 &&
-                           (in_dtype == AICOMP_KV_BF16 || in_dtype == AICOMP_KV_F32),
+                           (is_16bit_float(in_dtype) || in_dtype == AICOMP_KV_F32),
                        AICOMP_KV_EUNSUPPORTED,
-                       "kv_append: only f32/bf16 -> fp8 conversion is supported (in %d, pool %d)",
+                       "kv_append: only f32/bf16/f16 -> fp8 conversion is supported (in %d, pool %d)",
                        in_dtype, pool_dtype);
         AICOMP_REQUIRE(k_scale && v_scale, AICOMP_KV_EINVAL,
                        "kv_append: an fp8 pool needs k_scale and v_scale");
@@ -254,6 +259,11 @@ int launch_kv_append(const void* key, const void* value, int64_t token_stride, i
         if (in_dtype == AICOMP_KV_BF16)
             hipLaunchKernelGGL(kv_append_quant_fp8<bf16_t>, dim3((unsigned)blocks), dim3(threads), 0,
                                stream, (const bf16_t*)key, (const bf16_t*)value, token_stride,
+                               head_stride, (uint32_t*)k_pool, (uint32_t*)v_pool, slot_mapping,
+                               k_scale, v_scale, total, hkv, d / 4, bs, num_slots);
+        else if (in_dtype == AICOMP_KV_F16)
+            hipLaunchKernelGGL(kv_append_quant_fp8<f16_t>, dim3((unsigned)blocks), dim3(threads), 0,
+                               stream, (const f16_t*)key, (const f16_t*)value, token_stride,
                                head_stride, (uint32_t*)k_pool, (uint32_t*)v_pool, slot_mapping,
                                k_scale, v_scale, total, hkv, d / 4, bs, num_slots);
         else

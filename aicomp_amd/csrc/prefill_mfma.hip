@@ -19,17 +19,17 @@
 //              workgroups take their (chunk, query tile) items in order of cost, a long item
 //              and a short one side by side on a CU; otherwise the longest query tiles of
 //              every chunk are launched first.
-// K/V tiles    32 or 64 tokens per step, double-buffered in LDS, one barrier per tile.  bf16
-//              pools and two column groups: loaded straight into LDS
+// K/V tiles    32 or 64 tokens per step, double-buffered in LDS, one barrier per tile.  16-bit
+//              pools (bf16, fp16) and two column groups: loaded straight into LDS
 //              (global_load_lds_dwordx4, 1 KB = four or eight token rows per wave
 //              instruction) one tile ahead, rows unpadded with their 16-byte chunks
 //              XOR-swizzled by the row index.
 //              Otherwise: coalesced 16-byte loads into registers ahead of their use, written
-//              to LDS (one padded row per token; fp8 is widened to bf16 on the way).
+//              to LDS (one padded row per token; fp8 is widened to the query's type on the way).
 // head_dim     128 or 64, one instantiation each.
 // Per wave     16 or 32 rows (one or two column groups).  S^T = K Q^T with K rows as
 //              the A operand and the wave's query rows as B columns
-//              (v_mfma_f32_16x16x32_bf16); online softmax per column on the raw
+//              (v_mfma_f32_16x16x32_bf16 / _f16); online softmax per column on the raw
 //              scores with a lazily moved max: the exponentials are taken against the current
 //              max and their sum tells whether it has to move (then, rarely, the row max is
 //              found with two lane swaps and the exponentials are redone); O^T += V^T P^T
@@ -43,10 +43,6 @@
 #include <type_traits>
 
 namespace aicomp {
-
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 namespace {
 
@@ -70,22 +66,6 @@ struct PrefillParams {
     const float* k_scale;
     const float* v_scale;
 };
-
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-    bf16x2_t p = {(__bf16)lo, (__bf16)hi};
-    return __builtin_bit_cast(uint32_t, p);
-}
-
-__device__ __forceinline__ uint4 fp8x8_to_bf16x8(uint2 r) {
-    // gfx950 converts two e4m3 codes straight to two packed bf16 (exact: 3 mantissa bits);
-    // the scale operand is 1.0
-    uint4 o;
-    o.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.x, 1.0f, false));
-    o.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.x, 1.0f, true));
-    o.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.y, 1.0f, false));
-    o.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r.y, 1.0f, true));
-    return o;
-}
 
 // max over lanes l and l^16 (l^32): gfx950's lane-swap instructions, no LDS round trip.
 // v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of
@@ -115,17 +95,18 @@ template <int NL> struct Stage<true, NL> { uint2 k[NL], v[NL]; };
 // KT = rows of an LDS tile (KT/16 blocks): 32 with two register stages for R = 1, 64 with one stage
 // for R = 2, where the per-step work that does not scale with the tile (barrier, block lookups,
 // loop control, the running-max test) is paid half as often.
-// DMA = tiles go from the pool straight into LDS (bf16 pools, R = 2): no staging registers, no
+// DMA = tiles go from the pool straight into LDS (bf16 / fp16 pools, R = 2): no staging registers, no
 // LDS writes by the waves.  The two buffers are separate __shared__ arrays and every read address
 // is one offset from its array, which is what lets the compiler see that a read of one buffer
 // need not wait for the loads in flight into the other; the only wait is the explicit one at the
 // barrier that opens a step, for the loads issued one step earlier.
 #define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
-template <bool FP8, int R, int DH, bool DMA>
+// E = the 16-bit element format of queries, output and (unless FP8) the pools.
+template <typename E, bool FP8, int R, int DH, bool DMA>
 __global__ void __launch_bounds__(256, (R == 1 || DH == 64) ? 3 : 2)
 paged_prefill_mfma_kernel(PrefillParams p) {
-    static_assert(!DMA || (!FP8 && R == 2), "direct-to-LDS tiles: bf16 pools, two column groups");
+    static_assert(!DMA || (!FP8 && R == 2), "direct-to-LDS tiles: 16-bit pools, two column groups");
     constexpr int KROW = DMA ? 2 * DH : 2 * DH + 16;          // LDS row stride in bytes
     constexpr int NSL = DH / 32;               // 32-element k-slots of a row (QK^T MFMAs per 16 x 16 tile)
     constexpr int NJ = DH / 16;                // 16-element output tiles (PV MFMAs per 32 tokens)
@@ -243,13 +224,13 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     const int ntiles = (kv_end + TT - 1) / TT;
 
     // Q as the B operand: column = this lane's row, k-slots = dims 32s + 8*g4 ..
-    bf16x8_t qf[R][NSL];
+    uint4 qf[R][NSL];
 #pragma unroll
     for (int c = 0; c < R; ++c) {
-        const bf16_t* qrow = (const bf16_t*)p.query + ((int64_t)(q_begin + min(qpos[c], n - 1)) * p.hq + head[c]) * DH;
+        const uint16_t* qrow = (const uint16_t*)p.query + ((int64_t)(q_begin + min(qpos[c], n - 1)) * p.hq + head[c]) * DH;
 #pragma unroll
         for (int s = 0; s < NSL; ++s)                           // k-slot s, k-group g4: elements 32s + 8*g4 ..
-            qf[c][s] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(qrow + 32 * s + 8 * g4));
+            qf[c][s] = *(const uint4*)(qrow + 32 * s + 8 * g4);
     }
     // log2(e) * scale * k_scale.  The softmax below tracks the max of the raw scores, which needs
     // a positive multiplier: a negative one (a negative k_scale) moves its sign into Q.
@@ -260,9 +241,8 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         for (int c = 0; c < R; ++c)
 #pragma unroll
             for (int s = 0; s < NSL; ++s) {
-                uint4 u = __builtin_bit_cast(uint4, qf[c][s]);
-                u.x ^= 0x80008000u; u.y ^= 0x80008000u; u.z ^= 0x80008000u; u.w ^= 0x80008000u;
-                qf[c][s] = __builtin_bit_cast(bf16x8_t, u);
+                uint4& u = qf[c][s];
+                u.x ^= E::SIGN_PAIR; u.y ^= E::SIGN_PAIR; u.z ^= E::SIGN_PAIR; u.w ^= E::SIGN_PAIR;
             }
     }
 
@@ -326,7 +306,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             const int tok_local = RPL * i + tid / CPR;           // LDS row
             const int off = tok_local * KROW + (tid % CPR) * 16;
             uint4 kk, vv;
-            if constexpr (FP8) { kk = fp8x8_to_bf16x8(st.k[i]); vv = fp8x8_to_bf16x8(st.v[i]); }
+            if constexpr (FP8) { kk = E::from_fp8(st.k[i]); vv = E::from_fp8(st.v[i]); }
             else { kk = st.k[i]; vv = st.v[i]; }
             if constexpr (TAIL) {
                 if (t * KT + tok_local >= ctx) vv = make_uint4(0, 0, 0, 0);
@@ -438,18 +418,18 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             for (int c = 0; c < R; ++c) sa[h][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < NSL; ++s) {
-            bf16x8_t a[NH];
+            uint4 a[NH];
 #pragma unroll
             for (int h = 0; h < NH; ++h)
                 if constexpr (DMA)   // chunk 4s + g4 of row 16h + prow sits at chunk slot (4s + g4) ^ swz(prow)
-                    a[h] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kb + 16 * h * KROW + prow * KROW + (((4 * s + g4) ^ swz(prow)) << 4)));
+                    a[h] = *(const uint4*)(kb + 16 * h * KROW + prow * KROW + (((4 * s + g4) ^ swz(prow)) << 4));
                 else
-                    a[h] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kb + 16 * h * KROW + rd_k + s * 64));
+                    a[h] = *(const uint4*)(kb + 16 * h * KROW + rd_k + s * 64);
 #pragma unroll
             for (int h = 0; h < NH; ++h)
 #pragma unroll
                 for (int c = 0; c < R; ++c)
-                    sa[h][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[h], qf[c][s], sa[h][c], 0, 0, 0);
+                    sa[h][c] = E::mfma(a[h], qf[c][s], sa[h][c]);
         }
         // Online softmax on the raw scores: the score multiplier is folded into the exponent's
         // fused multiply-add and the running max stays in raw units.  The max is moved lazily:
@@ -457,7 +437,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         // them stays <= 2^8 every P is at most 256, exact enough in bf16 and f32, and neither the
         // max nor the accumulators are touched.  Only tiles that cross the diagonal pay for the mask.
         const bool need_mask = sub_start + TT - 1 > wave_kv_min;       // wave-uniform
-        bf16x8_t pf[R][NH / 2];
+        uint4 pf[R][NH / 2];
         float alpha[R];
         bool grew[R];                                                  // wave-uniform
         auto softmax = [&](auto mask_tag) {
@@ -490,10 +470,8 @@ paged_prefill_mfma_kernel(PrefillParams p) {
                         float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[k + 1], cmul, bias[c]));
                         if (MASK && dead[k]) p0 = 0.f;
                         if (MASK && dead[k + 1]) p1 = 0.f;
-                        const bf16x2_t pp = {(__bf16)p0, (__bf16)p1};
-                        const bf16x2_t one = {(__bf16)1.0f, (__bf16)1.0f};
-                        psum = __builtin_amdgcn_fdot2_f32_bf16(pp, one, psum, false);
-                        pk[k >> 1] = __builtin_bit_cast(uint32_t, pp);
+                        pk[k >> 1] = E::pack(p0, p1);
+                        psum = E::pair_sum(pk[k >> 1], psum);
                     }
                 };
                 exps();
@@ -521,7 +499,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
                 for (int hp = 0; hp < NH / 2; ++hp) {
                     uint4 pw;
                     pw.x = pk[4 * hp + 0]; pw.y = pk[4 * hp + 1]; pw.z = pk[4 * hp + 2]; pw.w = pk[4 * hp + 3];
-                    pf[c][hp] = __builtin_bit_cast(bf16x8_t, pw);
+                    pf[c][hp] = pw;
                 }
             }
         };
@@ -552,10 +530,10 @@ paged_prefill_mfma_kernel(PrefillParams p) {
                 const v4i16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(vb + voff));
                 const v4i16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(vb + (voff + 16 * KROW)));
                 const v8i16_t av = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                const bf16x8_t a = __builtin_bit_cast(bf16x8_t, av);
+                const uint4 a = __builtin_bit_cast(uint4, av);
 #pragma unroll
                 for (int c = 0; c < R; ++c)
-                    O[c][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[c][hp], O[c][j], 0, 0, 0);
+                    O[c][j] = E::mfma(a, pf[c][hp], O[c][j]);
             }
         }
     };
@@ -592,16 +570,16 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         l += __shfl_xor(l, 32);
         if (row_valid[c]) {
             const float inv = (l > 0.f ? 1.f / l : 0.f) * (FP8 ? p.v_scale[kvh] : 1.f);
-            bf16_t* o = (bf16_t*)p.out + ((int64_t)(q_begin + qpos[c]) * p.hq + head[c]) * DH + 4 * g4;
+            uint16_t* o = (uint16_t*)p.out + ((int64_t)(q_begin + qpos[c]) * p.hq + head[c]) * DH + 4 * g4;
 #pragma unroll
             for (int j = 0; j < NJ; ++j)
-                *(uint2*)(o + 16 * j) = make_uint2(pack_bf16(O[c][j][0] * inv, O[c][j][1] * inv),
-                                                   pack_bf16(O[c][j][2] * inv, O[c][j][3] * inv));
+                *(uint2*)(o + 16 * j) = make_uint2(E::pack(O[c][j][0] * inv, O[c][j][1] * inv),
+                                                   E::pack(O[c][j][2] * inv, O[c][j][3] * inv));
         }
     }
 }
 
-template <bool FP8, int R, int DH, bool DMA = false>
+template <typename E, bool FP8, int R, int DH, bool DMA = false>
 static hipError_t launch_prefill_variant(const PrefillParams& p, dim3 grid, size_t lds_bytes, hipStream_t stream) {
     // Two column groups stage 64-row tiles: 70 KB of dynamic LDS, above the 64 KB a kernel may use
     // without asking.  The limit is a per-device function attribute: set once per device.
@@ -611,12 +589,12 @@ static hipError_t launch_prefill_variant(const PrefillParams& p, dim3 grid, size
     if (e != hipSuccess) return e;
     const bool known = dev < 64 && ((done.load(std::memory_order_acquire) >> dev) & 1ull);
     if (!known) {
-        e = hipFuncSetAttribute((const void*)paged_prefill_mfma_kernel<FP8, R, DH, DMA>,
+        e = hipFuncSetAttribute((const void*)paged_prefill_mfma_kernel<E, FP8, R, DH, DMA>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return e;
         if (dev < 64) done.fetch_or(1ull << dev, std::memory_order_release);
     }
-    hipLaunchKernelGGL((paged_prefill_mfma_kernel<FP8, R, DH, DMA>), grid, dim3(256), lds_bytes, stream, p);
+    hipLaunchKernelGGL((paged_prefill_mfma_kernel<E, FP8, R, DH, DMA>), grid, dim3(256), lds_bytes, stream, p);
     return hipSuccess;
 }
 
@@ -625,8 +603,8 @@ static hipError_t launch_prefill_variant(const PrefillParams& p, dim3 grid, size
 bool prefill_mfma_supported(const DecodeArgs& a, int max_q_len) {
     const int group = a.hkv > 0 ? a.hq / a.hkv : 0;
     return a.cu_q_lens != nullptr && max_q_len > 0 && (a.d == 128 || a.d == 64) && a.bs == BS &&
-           a.q_dtype == AICOMP_KV_BF16 &&
-           (a.kv_dtype == AICOMP_KV_BF16 || a.kv_dtype == AICOMP_KV_FP8_E4M3) && group >= 1 &&
+           is_16bit_float(a.q_dtype) &&
+           (a.kv_dtype == a.q_dtype || a.kv_dtype == AICOMP_KV_FP8_E4M3) && group >= 1 &&
            a.scale > 0.f && a.num_seqs <= 65535 && ((uintptr_t)a.query % 16 == 0) &&
            ((uintptr_t)a.out % 16 == 0) && ((uintptr_t)a.k_pool % 16 == 0) &&
            ((uintptr_t)a.v_pool % 16 == 0);
@@ -666,17 +644,23 @@ int launch_prefill_mfma(const DecodeArgs& a, int max_q_len) {
     const size_t lds_bytes = (size_t)4 * (R == 1 ? 32 : 64) * (2 * a.d + 16);
     const bool fp8 = a.kv_dtype == AICOMP_KV_FP8_E4M3;
     hipError_t e;
-    if (a.d == 64) {
-        if (fp8 && R == 2) e = launch_prefill_variant<true, 2, 64>(p, grid, lds_bytes, a.stream);
-        else if (fp8) e = launch_prefill_variant<true, 1, 64>(p, grid, lds_bytes, a.stream);
-        else if (R == 2) e = launch_prefill_variant<false, 2, 64, true>(p, grid, 0, a.stream);    // static LDS
-        else e = launch_prefill_variant<false, 1, 64>(p, grid, lds_bytes, a.stream);
-    } else {
-        if (fp8 && R == 2) e = launch_prefill_variant<true, 2, 128>(p, grid, lds_bytes, a.stream);
-        else if (fp8) e = launch_prefill_variant<true, 1, 128>(p, grid, lds_bytes, a.stream);
-        else if (R == 2) e = launch_prefill_variant<false, 2, 128, true>(p, grid, 0, a.stream);   // static LDS
-        else e = launch_prefill_variant<false, 1, 128>(p, grid, lds_bytes, a.stream);
-    }
+#define AICOMP_LAUNCH_PREFILL(E)                                                                                      \
+    do {                                                                                                              \
+        if (a.d == 64) {                                                                                              \
+            if (fp8 && R == 2) e = launch_prefill_variant<E, true, 2, 64>(p, grid, lds_bytes, a.stream);              \
+            else if (fp8) e = launch_prefill_variant<E, true, 1, 64>(p, grid, lds_bytes, a.stream);                   \
+            else if (R == 2) e = launch_prefill_variant<E, false, 2, 64, true>(p, grid, 0, a.stream);  /* static LDS */ \
+            else e = launch_prefill_variant<E, false, 1, 64>(p, grid, lds_bytes, a.stream);                           \
+        } else {                                                                                                      \
+            if (fp8 && R == 2) e = launch_prefill_variant<E, true, 2, 128>(p, grid, lds_bytes, a.stream);             \
+            else if (fp8) e = launch_prefill_variant<E, true, 1, 128>(p, grid, lds_bytes, a.stream);                  \
+            else if (R == 2) e = launch_prefill_variant<E, false, 2, 128, true>(p, grid, 0, a.stream); /* static LDS */ \
+            else e = launch_prefill_variant<E, false, 1, 128>(p, grid, lds_bytes, a.stream);                          \
+        }                                                                                                             \
+    } while (0)
+    if (a.q_dtype == AICOMP_KV_F16) AICOMP_LAUNCH_PREFILL(F16Fmt);
+    else AICOMP_LAUNCH_PREFILL(Bf16Fmt);
+#undef AICOMP_LAUNCH_PREFILL
     AICOMP_REQUIRE(e == hipSuccess, AICOMP_KV_EHIP, "paged_prefill_attn: %s", hipGetErrorString(e));
     AICOMP_HIP_LAUNCH_CHECK();
     return AICOMP_KV_OK;

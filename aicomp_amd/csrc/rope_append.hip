@@ -58,6 +58,16 @@ template <> struct Row8<bf16_t> {
     // value as the tensor type holds it
     __device__ __forceinline__ static float round(float v) { return (float)(__bf16)v; }
 };
+template <> struct Row8<f16_t> {
+    __device__ __forceinline__ static void load(const f16_t* p, float* f) {
+        Vec16<f16_t>::unpack(*(const uint4*)p, f);
+    }
+    __device__ __forceinline__ static void store(f16_t* p, const float* f) {
+        *(uint4*)p = make_uint4(F16Fmt::pack(f[0], f[1]), F16Fmt::pack(f[2], f[3]), F16Fmt::pack(f[4], f[5]),
+                                F16Fmt::pack(f[6], f[7]));
+    }
+    __device__ __forceinline__ static float round(float v) { return (float)(_Float16)v; }
+};
 template <> struct Row8<float> {
     __device__ __forceinline__ static void load(const float* p, float* f) {
         const float4 a = ((const float4*)p)[0], b = ((const float4*)p)[1];
@@ -203,6 +213,9 @@ int launch_rope_kv_append(const void* q_in, void* q_out, int64_t q_ts, int64_t q
     if (in_dtype == AICOMP_KV_BF16) {
         if (fp8) hipLaunchKernelGGL((rope_kv_append_kernel<bf16_t, true>), grid, block, 0, stream, p);
         else hipLaunchKernelGGL((rope_kv_append_kernel<bf16_t, false>), grid, block, 0, stream, p);
+    } else if (in_dtype == AICOMP_KV_F16) {
+        if (fp8) hipLaunchKernelGGL((rope_kv_append_kernel<f16_t, true>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((rope_kv_append_kernel<f16_t, false>), grid, block, 0, stream, p);
     } else {
         if (fp8) hipLaunchKernelGGL((rope_kv_append_kernel<float, true>), grid, block, 0, stream, p);
         else hipLaunchKernelGGL((rope_kv_append_kernel<float, false>), grid, block, 0, stream, p);

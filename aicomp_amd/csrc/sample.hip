@@ -28,6 +28,8 @@
 // share the leading key bits.
 #include "common.h"
 
+#include <type_traits>
+
 namespace aicomp {
 
 namespace {
@@ -78,7 +80,13 @@ __device__ __forceinline__ float scaled_logit<bf16_t>(const bf16_t* row, int i, 
     return temperature == 1.f ? x : (float)(__bf16)(x / temperature);
 }
 
-// four consecutive logits in one load (16 bytes of fp32, 8 bytes of bf16)
+template <>
+__device__ __forceinline__ float scaled_logit<f16_t>(const f16_t* row, int i, float temperature) {
+    const float x = f16_to_f32(row[i].bits);
+    return temperature == 1.f ? x : (float)(_Float16)(x / temperature);
+}
+
+// four consecutive logits in one load (16 bytes of fp32, 8 bytes of bf16 / fp16)
 template <typename T> struct Load4;
 template <> struct Load4<float> {
     __device__ __forceinline__ static void get(const float* p, float* x) {
@@ -93,12 +101,34 @@ template <> struct Load4<bf16_t> {
         x[2] = __uint_as_float(v.y << 16); x[3] = __uint_as_float(v.y & 0xffff0000u);
     }
 };
+template <> struct Load4<f16_t> {
+    __device__ __forceinline__ static void get(const f16_t* p, float* x) {
+        const uint2 v = *(const uint2*)p;
+        x[0] = f16_to_f32((uint16_t)(v.x & 0xffffu)); x[1] = f16_to_f32((uint16_t)(v.x >> 16));
+        x[2] = f16_to_f32((uint16_t)(v.y & 0xffffu)); x[3] = f16_to_f32((uint16_t)(v.y >> 16));
+    }
+};
+// For fp16 rows: a raw value below which the scaled, rounded logit is certainly below `q_scaled`.
+// A quotient rounds up by at most half a unit in the last place of the result, 2^-25 in fp16's
+// subnormal range, so everything from q - max(2^-24, |q| 2^-10) up may still reach q; the
+// float division adds a relative 2^-24.  Other types: +inf (no extra lowering).
+template <typename T> __device__ __forceinline__ float f16_raw_bound(float q_scaled, float temperature) {
+    if constexpr (std::is_same<T, f16_t>::value) {
+        const float y = (q_scaled - fmaxf(5.9604645e-8f, fabsf(q_scaled) * 9.765625e-4f)) * temperature;
+        return y - fabsf(y) * 9.5367431640625e-7f;
+    } else {
+        return __builtin_inff();
+    }
+}
 template <typename T> __device__ __forceinline__ float apply_temperature(float x, float temperature);
 template <> __device__ __forceinline__ float apply_temperature<float>(float x, float temperature) {
     return temperature == 1.f ? x : x / temperature;
 }
 template <> __device__ __forceinline__ float apply_temperature<bf16_t>(float x, float temperature) {
     return temperature == 1.f ? x : (float)(__bf16)(x / temperature);
+}
+template <> __device__ __forceinline__ float apply_temperature<f16_t>(float x, float temperature) {
+    return temperature == 1.f ? x : (float)(_Float16)(x / temperature);
 }
 
 // f(index, scaled logit) over the elements [begin, end) owned by `rank` of `nranks` lanes.
@@ -467,7 +497,7 @@ sample_kernel(SampleParams p) {
         // prefilter on the raw float, one compare per element.  It lets through whatever the key
         // order would (plus -0.0 next to +0.0, and everything when the bound is below -inf, whose
         // key decodes to a NaN); the exact test on the scaled key follows.
-        const float raw_lo = key_value(key_lo);
+        const float raw_lo = fminf(key_value(key_lo), f16_raw_bound<T>(key_value(key_ls), temp));
         for_each_logit<T>(row, 0, V, 1.f, tid, NT, vec_ok, [&](int i, float x) {
             if (!(x < raw_lo)) {
                 const uint32_t key = order_key(apply_temperature<T>(x, temp));
@@ -616,8 +646,9 @@ sample_kernel(SampleParams p) {
                 // raw prefilter: the scaled bound times the temperature, lowered by more than the division
                 // (and, for bf16 rows, the rounding of the quotient) can move a value
                 const float t_raw = key_value(key_lo_s) * temp;
-                const float raw_lo = temp == 1.f ? key_value(key_lo_s)
-                                                 : t_raw - fabsf(t_raw) * (sizeof(T) == 2 ? 0.0078125f : 9.5367431640625e-7f);
+                const float raw_lo = fminf(temp == 1.f ? key_value(key_lo_s)
+                                                       : t_raw - fabsf(t_raw) * (sizeof(T) == 2 ? 0.0078125f : 9.5367431640625e-7f),
+                                           f16_raw_bound<T>(key_value(key_lo_s), temp));
                 for_each_logit<T>(row, 0, V, 1.f, tid, NT, vec_ok, [&](int i, float x) {
                     if (!(x < raw_lo)) {
                         const uint32_t key = order_key(apply_temperature<T>(x, temp));
@@ -870,6 +901,7 @@ int launch_sample(int64_t* out, const void* logits, int64_t row_stride, float* p
     p.uniforms = uniforms; p.vocab = vocab; p.temperature = temperature; p.top_k = top_k;
     p.top_p = top_p; p.greedy = greedy;
     if (dtype == AICOMP_KV_F32) hipLaunchKernelGGL((sample_kernel<float>), dim3(batch), dim3(NT), 0, stream, p);
+    else if (dtype == AICOMP_KV_F16) hipLaunchKernelGGL((sample_kernel<f16_t>), dim3(batch), dim3(NT), 0, stream, p);
     else hipLaunchKernelGGL((sample_kernel<bf16_t>), dim3(batch), dim3(NT), 0, stream, p);
     AICOMP_HIP_LAUNCH_CHECK();
     return AICOMP_KV_OK;

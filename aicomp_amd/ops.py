@@ -14,14 +14,15 @@ import torch
 
 from . import _lib
 
-_DT = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float8_e4m3fn: _lib.FP8_E4M3}
+_DT = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16,
+       torch.float8_e4m3fn: _lib.FP8_E4M3}
 
 
 def _dt(t: torch.Tensor, what: str) -> int:
     try:
         return _DT[t.dtype]
     except KeyError:
-        raise RuntimeError(f"{what}: unsupported dtype {t.dtype} (float32, bfloat16, float8_e4m3fn)")
+        raise RuntimeError(f"{what}: unsupported dtype {t.dtype} (float32, bfloat16, float16, float8_e4m3fn)")
 
 
 def _req(cond: bool, msg: str) -> None:
@@ -345,7 +346,7 @@ def rope_kv_append(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, 
          f"key/value {tuple(key.shape)} and query {tuple(query.shape)} do not match pools {tuple(k_pool.shape)}")
     _req(key.dtype == query.dtype and value.dtype == query.dtype and out.dtype == query.dtype,
          "query, key, value and query_out must share one dtype")
-    _req(query.dtype in (torch.float32, torch.bfloat16), f"unsupported input dtype {query.dtype}")
+    _req(query.dtype in (torch.float32, torch.bfloat16, torch.float16), f"unsupported input dtype {query.dtype}")
     for t, n in ((query, "query"), (out, "query_out"), (key, "key"), (value, "value")):
         _req(t.stride(2) == 1, f"{n}: last dimension must be contiguous")
     _req(key.stride() == value.stride(), "key and value must have equal strides")
@@ -391,7 +392,7 @@ def sample_tokens(logits: torch.Tensor, temperature: float = 1.0, top_k: int = 0
     lib = _lib.load()
     _req(logits.is_cuda, "tensors must live on a ROCm device (there is no CPU path)")
     _req(logits.dim() == 2 and logits.stride(1) == 1, "logits must be [B, V] with contiguous rows")
-    _req(logits.dtype in (torch.float32, torch.bfloat16), f"unsupported logits dtype {logits.dtype}")
+    _req(logits.dtype in (torch.float32, torch.bfloat16, torch.float16), f"unsupported logits dtype {logits.dtype}")
     B, V = logits.shape
     out = torch.empty(B, dtype=torch.int64, device=logits.device)
     probs = torch.empty(B, V, dtype=torch.float32, device=logits.device) if return_probs else None

@@ -44,6 +44,7 @@ extern "C" {
 #define AICOMP_KV_F32       0
 #define AICOMP_KV_BF16      1
 #define AICOMP_KV_FP8_E4M3  2       /* OCP e4m3 ("e4m3fn"), max finite 448       */
+#define AICOMP_KV_F16       3       /* IEEE binary16                             */
 
 /* Library version (major*10000 + minor*100 + patch). */
 int aicomp_kv_version(void);
@@ -63,8 +64,8 @@ const char* aicomp_kv_last_error(void);
  *                  or >= num_blocks * block_size (outside the pool) is skipped without an error:
  *                  the library cannot report a per-row fault from a kernel, so a planner that
  *                  wants to hear about such rows checks its slots on the host
- *   in_dtype == pool_dtype                  raw copy, bit-exact
- *   in_dtype f32/bf16, pool_dtype FP8_E4M3  code = e4m3_rne(clamp(x / scale[h], +-448)),
+ *   in_dtype == pool_dtype                  raw copy, bit-exact (F32, BF16, F16, FP8_E4M3)
+ *   in_dtype f32/bf16/f16, pool FP8_E4M3    code = e4m3_rne(clamp(x / scale[h], +-448)),
  *                                           k_scale / v_scale [Hkv] float, required
  */
 int aicomp_kv_append(const void* key, const void* value,
@@ -82,7 +83,8 @@ int aicomp_kv_append(const void* key, const void* value,
  * full_value, attn_mask=None, is_causal=False)   (kv_cache.py:397-403)
  * including the .contiguous() prefix copies it is fed from (kv_cache.py:391-392).
  *
- *   out, query      [B, Hq, D] of q_dtype, contiguous
+ *   out, query      [B, Hq, D] of q_dtype (F32, BF16 or F16), contiguous; the pools hold
+ *                   kv_dtype == q_dtype, or FP8_E4M3 under BF16 / F16 queries
  *   block_table     [B, max_blocks_per_seq] int32, row stride block_table_stride.  Entries are
  *                   trusted to lie in [0, num_blocks); one that does not is clamped into the
  *                   pool (no fault, and no error: the row then attends over another block)
@@ -195,12 +197,12 @@ int aicomp_paged_decode_partition_size(int batch, int num_q_heads, int num_kv_he
                                        int max_blocks_per_seq, int q_dtype, int kv_dtype);
 
 /*
- * Chunked-prefill causal attention over the paged pool (MFMA bf16).
+ * Chunked-prefill causal attention over the paged pool (matrix cores for bf16 and fp16).
  * Replaces the prefill branch  F.scaled_dot_product_attention(query, full_key,
  * full_value, attn_mask=None, is_causal=True)   (kv_cache.py:404-415).
  * The chunk's own K/V rows must already be in the pool (append first).
  *
- *   out, query     [T, Hq, D] bf16, rows of sequence s are cu_q_lens[s]..cu_q_lens[s+1]
+ *   out, query     [T, Hq, D] of q_dtype, rows of sequence s are cu_q_lens[s]..cu_q_lens[s+1]
  *   context_lens   [S] int32: prior context + chunk length
  *   cu_q_lens      [S+1] int32 prefix sums of the chunk lengths
  *   max_q_len      host-side upper bound of the chunk lengths (sizes the grid)
@@ -227,7 +229,7 @@ int aicomp_paged_prefill_attn(void* out, const void* query,
  * and the append of k_embed / value                (kv_cache.py:387-388), with the KV heads
  * stored once instead of repeat_kv's G copies      (modeling_llama.py:268-277, :589-590).
  *
- *   q_in, q_out     [T, Hq, D] of in_dtype (F32 or BF16); element (t,h,d) at
+ *   q_in, q_out     [T, Hq, D] of in_dtype (F32, BF16 or F16); element (t,h,d) at
  *                   t*token_stride + h*head_stride + d of the respective stride pair;
  *                   q_out may be q_in (in place)
  *   key, value      [T, Hkv, D] of in_dtype, strides as in aicomp_kv_append (the three inputs
@@ -266,7 +268,7 @@ int aicomp_rope_kv_append(const void* q_in, void* q_out,
  * then a draw from the softmax of what is left (:840-841).
  *
  *   out           [B] int64 token ids
- *   logits        [B, V] F32 or BF16, row b at b*row_stride elements; not modified
+ *   logits        [B, V] F32, BF16 or F16, row b at b*row_stride elements; not modified
  *   uniforms      [B] float in [0, 1): the draw is the inverse CDF in index order at
  *                 uniforms[b] (the reference draws with torch.multinomial; the distribution is
  *                 the same, the random stream is the caller's).  Not read when greedy.

@@ -41,6 +41,8 @@ PARITY PINNING STATUS
   is "parity unpinned": none exist for this path.
 * fp8 e4m3 (not in the reference): pinned against torch's ``float8_e4m3fn``
   cast over all 256 codes and on random data.
+* bf16 / fp16 codecs: pinned against torch's casts over all 65 536 codes (decode) and on
+  random data, ties, overflow and subnormals (encode).
 """
 from __future__ import annotations
 
@@ -70,6 +72,26 @@ def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
     out = rounded.astype(np.uint16)
     out[nan] = ((u[nan] >> np.uint32(16)) | np.uint32(0x0040)).astype(np.uint16)
     return out
+
+
+def f16_bits_to_f32(bits: np.ndarray) -> np.ndarray:
+    """uint16 IEEE binary16 codes -> float32 (exact): 1 sign, 5 exponent (bias 15), 10 mantissa;
+    exponent 0 is subnormal (m * 2^-24), exponent 31 is inf / NaN."""
+    b = np.asarray(bits, dtype=np.uint16).astype(np.int64)
+    sign = np.where(b & 0x8000, -1.0, 1.0)
+    e = (b >> 10) & 0x1F
+    m = b & 0x3FF
+    with np.errstate(invalid="ignore"):
+        v = np.where(e == 0, m * 2.0 ** -24, (1.0 + m / 1024.0) * np.exp2((e - 15).astype(np.float64)))
+        v = np.where(e == 31, np.where(m == 0, np.inf, np.nan), v)
+    return (sign * v).astype(np.float32)
+
+
+def f32_to_f16_bits(x: np.ndarray) -> np.ndarray:
+    """float32 -> uint16 binary16 codes, round to nearest even, overflow to infinity (numpy's
+    conversion; pinned against torch's cast in the tests)."""
+    with np.errstate(over="ignore"):
+        return np.asarray(x, dtype=np.float32).astype(np.float16).view(np.uint16)
 
 
 def e4m3_code_table() -> np.ndarray:
@@ -123,11 +145,13 @@ def f32_to_e4m3_bits(x: np.ndarray) -> np.ndarray:
 
 
 def decode_elements(raw: np.ndarray, dtype: str) -> np.ndarray:
-    """Raw storage array -> float64 values.  dtype in {"f32","bf16","fp8"}."""
+    """Raw storage array -> float64 values.  dtype in {"f32","bf16","f16","fp8"}."""
     if dtype == "f32":
         return np.asarray(raw, dtype=np.float32).astype(np.float64)
     if dtype == "bf16":
         return bf16_bits_to_f32(raw).astype(np.float64)
+    if dtype == "f16":
+        return f16_bits_to_f32(raw).astype(np.float64)
     if dtype == "fp8":
         return e4m3_bits_to_f32(raw).astype(np.float64)
     raise ValueError(dtype)

@@ -61,11 +61,13 @@ def rope_angles(inv_freq: np.ndarray, positions: Sequence[int]) -> np.ndarray:
 
 
 def _to_type(x32: np.ndarray, dtype: str) -> np.ndarray:
-    """float32 values -> storage codes of ``dtype`` ("f32": float32, "bf16": uint16 bits)."""
+    """float32 values -> storage codes of ``dtype`` ("f32": float32, "bf16" / "f16": uint16 bits)."""
     if dtype == "f32":
         return x32.astype(np.float32)
     if dtype == "bf16":
         return P.f32_to_bf16_bits(x32.astype(np.float32))
+    if dtype == "f16":
+        return P.f32_to_f16_bits(x32.astype(np.float32))
     raise ValueError(dtype)
 
 
@@ -74,6 +76,8 @@ def _to_f32(raw: np.ndarray, dtype: str) -> np.ndarray:
         return np.asarray(raw, dtype=np.float32)
     if dtype == "bf16":
         return P.bf16_bits_to_f32(np.asarray(raw, dtype=np.uint16))
+    if dtype == "f16":
+        return P.f16_bits_to_f32(np.asarray(raw, dtype=np.uint16))
     raise ValueError(dtype)
 
 

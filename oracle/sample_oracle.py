@@ -44,6 +44,8 @@ def scaled(logits_row: np.ndarray, temperature: float, dtype: str = "f32") -> np
         x = (x / np.float32(temperature)).astype(np.float32)
         if dtype == "bf16":
             x = P.bf16_bits_to_f32(P.f32_to_bf16_bits(x))
+        elif dtype == "f16":
+            x = P.f16_bits_to_f32(P.f32_to_f16_bits(x))
     return x
 
 

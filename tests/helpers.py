@@ -2,15 +2,15 @@
 import numpy as np
 import torch
 
-NAME = {torch.float32: "f32", torch.bfloat16: "bf16", torch.float8_e4m3fn: "fp8"}
+NAME = {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16", torch.float8_e4m3fn: "fp8"}
 
 
 def raw(t: torch.Tensor) -> np.ndarray:
-    """Tensor -> numpy array of its storage codes (f32 / uint16 / uint8)."""
+    """Tensor -> numpy array of its storage codes (f32 / uint16 for bf16 and fp16 / uint8)."""
     t = t.detach().cpu().contiguous()
     if t.dtype == torch.float32:
         return t.numpy()
-    if t.dtype == torch.bfloat16:
+    if t.dtype in (torch.bfloat16, torch.float16):
         return t.view(torch.int16).numpy().view(np.uint16)
     if t.dtype == torch.float8_e4m3fn:
         return t.view(torch.uint8).numpy()

@@ -97,7 +97,7 @@ def test_rope_refusals(lib):
     assert call(tokens=0) == 0
     assert call(q_in=None) == EINVAL and "null pointer" in err(lib)
     assert call(table_rows=0) == EINVAL
-    assert call(in_dtype=FP8) == EUNSUPPORTED and "float32 or bfloat16" in err(lib)
+    assert call(in_dtype=FP8) == EUNSUPPORTED and "float32, bfloat16 or float16" in err(lib)
     assert call(pool_dtype=F32) == EUNSUPPORTED                      # bf16 input, fp32 pool
     assert call(pool_dtype=FP8) == EINVAL and "k_scale" in err(lib)
     assert call(d=72) == EUNSUPPORTED and "multiple of 16" in err(lib)

@@ -16,7 +16,7 @@ def check_rows(device, x_cpu, temperature, top_k, top_p, dtype=torch.float32, se
     g = torch.Generator().manual_seed(seed)
     u = torch.rand(B, generator=g)
     xt = torch.from_numpy(x_cpu).to(dtype)
-    name = "bf16" if dtype == torch.bfloat16 else "f32"
+    name = {torch.bfloat16: "bf16", torch.float16: "f16"}.get(dtype, "f32")
     vals = xt.float().numpy()
     tok, probs = ops.sample_tokens(xt.to(device), temperature, top_k, top_p, True, u.to(device), return_probs=True)
     torch.cuda.synchronize()

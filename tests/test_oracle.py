@@ -34,6 +34,32 @@ def test_bf16_encode_rne_matches_torch():
     assert np.array_equal(got, want)
 
 
+def test_f16_decode_all_codes_match_torch():
+    codes = np.arange(65536, dtype=np.uint16)
+    want = torch.from_numpy(codes.view(np.int16)).view(torch.float16).float().numpy()
+    got = orc.f16_bits_to_f32(codes)
+    assert np.array_equal(got.view(np.uint32)[~np.isnan(want)], want.view(np.uint32)[~np.isnan(want)])
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+
+
+def test_f16_encode_rne_matches_torch():
+    g = torch.Generator().manual_seed(2)
+    x = torch.cat([torch.randn(200000, generator=g) * 10, torch.randn(50000, generator=g) * 1e-6,
+                   torch.randn(20000, generator=g) * 3e4])
+    # ties (even and odd neighbours), the overflow threshold, the subnormal range, signed zeros
+    ties = torch.tensor([1.0 + 2 ** -11, 1.0 + 3 * 2 ** -11, -1.0 - 2 ** -11, 65504.0, 65519.99, 65520.0, 7e4,
+                         2 ** -24, 2 ** -25, 1.5 * 2 ** -25, 3 * 2 ** -25, 6.0e-5, 6.1e-5, 0.0, -0.0,
+                         float("inf"), -float("inf"), 1e-10])
+    x = torch.cat([x, ties])
+    want = raw(x.to(torch.float16))
+    got = orc.f32_to_f16_bits(x.numpy())
+    assert np.array_equal(got, want)
+    # and back: every finite code survives a round trip
+    codes = np.arange(65536, dtype=np.uint16)
+    finite = ((codes >> 10) & 0x1F) != 31
+    assert np.array_equal(orc.f32_to_f16_bits(orc.f16_bits_to_f32(codes[finite])), codes[finite])
+
+
 def test_e4m3_table_matches_torch_all_codes():
     codes = torch.arange(256, dtype=torch.uint8)
     want = codes.view(torch.float8_e4m3fn).float().numpy()
