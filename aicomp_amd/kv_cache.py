@@ -132,12 +132,11 @@ class _PagedLayer:
     def attend(self, query: torch.Tensor, pos: int, scale: float) -> torch.Tensor:
         """query ``[B, Hq, n, D]`` at positions pos..pos+n (rows already appended)."""
         B, Hq, n, D = query.shape
-        self.context_lens.fill_(pos + n)
+        ctx = self.ctx_rows[pos + n]              # every sequence sees pos + n tokens: a row view, no fill launch
         if n == 1:
             q = query[:, :, 0, :].contiguous()
             out = torch.empty_like(q)
-            ops.paged_decode_attn(out, q, self.k_pool, self.v_pool, self.block_table,
-                                  self.context_lens, scale)
+            ops.paged_decode_attn(out, q, self.k_pool, self.v_pool, self.block_table, ctx, scale)
             return out.view(B, Hq, 1, D)
         if self._cu_n != n:
             self.cu_q_lens.copy_(torch.arange(B + 1, dtype=torch.int32, device=query.device) * n)
@@ -146,7 +145,7 @@ class _PagedLayer:
         q = query.permute(0, 2, 1, 3).reshape(B * n, Hq, D).contiguous()
         out = torch.empty_like(q)
         ops.paged_prefill_attn(out, q, self.k_pool, self.v_pool, self.block_table,
-                               self.context_lens, self.cu_q_lens, scale, max_q_len=n)
+                               ctx, self.cu_q_lens, scale, max_q_len=n)
         return out.view(B, n, Hq, D).permute(0, 2, 1, 3)
 
     def gather(self, end: int, heads: int) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -237,9 +236,9 @@ class KVCacheManager:
                              f"(range: {self.layer_start}-{self.layer_end})")
         return self._cache[layer_idx]
 
-    def append(self, layer_idx: int, new_k: torch.Tensor, new_v: torch.Tensor,
-               position: Optional[int] = None) -> Tuple[_PagedLayer, int, int]:
-        """The storage half of ``update``: returns (layer store, start, end)."""
+    def _place(self, layer_idx: int, new_k: torch.Tensor, new_v: torch.Tensor, position: Optional[int]):
+        """The checks and shape rules of ``update`` (``kv_cache.py:132-156``): unknown layer and
+        overflow raise ``ValueError``, 3-D input is batch 1, batch 1 broadcasts over the batch."""
         layer = self._layer(layer_idx)
         if position is None:
             position = self._seq_len
@@ -252,10 +251,35 @@ class KVCacheManager:
         if end_position > self.max_seq_len:
             raise ValueError(f"Cache overflow: position {position} + new_seq_len {new_k.size(2)} "
                              f"> max_seq_len {self.max_seq_len}")
-        layer.append(new_k, new_v, position, self.group)
+        return layer, new_k, new_v, position, end_position
+
+    def _advance(self, layer_idx: int, end_position: int) -> None:
+        # only the stage's first layer moves the shared length (kv_cache.py:163-164)
         if layer_idx == self.layer_start:
             self._seq_len = max(self._seq_len, end_position)
+
+    def append(self, layer_idx: int, new_k: torch.Tensor, new_v: torch.Tensor,
+               position: Optional[int] = None) -> Tuple[_PagedLayer, int, int]:
+        """The storage half of ``update``: returns (layer store, start, end)."""
+        layer, new_k, new_v, position, end_position = self._place(layer_idx, new_k, new_v, position)
+        layer.append(new_k, new_v, position, self.group)
+        self._advance(layer_idx, end_position)
         return layer, position, end_position
+
+    def decode_step(self, layer_idx: int, query: torch.Tensor, new_k: torch.Tensor, new_v: torch.Tensor,
+                    position: Optional[int], scale: float) -> Optional[torch.Tensor]:
+        """``update`` of one new token per sequence and the attention over the result in ONE library
+        call (the fused append + decode entry point), with ``update``'s checks and length rule.
+        Returns ``None`` when the step is not of that form (more than one token, or rows that need a
+        type conversion): the caller then appends and attends separately."""
+        if new_k.size(-2) != 1:
+            return None
+        layer, new_k, new_v, position, end_position = self._place(layer_idx, new_k, new_v, position)
+        if new_k.dtype != layer.k_pool.dtype or query.size(0) != layer.batch:
+            return None
+        out = layer.decode_step(query, new_k, new_v, position, self.group, scale)
+        self._advance(layer_idx, end_position)
+        return out
 
     def update(self, layer_idx: int, new_k: torch.Tensor, new_v: torch.Tensor,
                position: Optional[int] = None) -> Tuple[PagedKVView, PagedKVView]:
@@ -378,6 +402,11 @@ class CachedScaledDotProductAttention(nn.Module):
         if self.kv_manager is not None:
             # external mode (kv_cache.py:356-368): storage belongs to the manager; the explicit
             # position keeps several layers of one forward pass on the same write position
+            if n == 1:                            # decode step: one fused call, as in internal mode
+                out = self.kv_manager.decode_step(self.layer_idx, query, key, value, pos, scale)
+                if out is not None:
+                    self.cache_pos = pos + 1
+                    return out
             store, _, _ = self.kv_manager.append(self.layer_idx, key, value, position=pos)
         else:
             if self._store is None:

@@ -149,3 +149,62 @@ def test_adapter_batch_one_and_hf_style_views(device):
     err = (got.float().cpu() - want).abs()
     assert bool(((err <= 1e-2) | (err <= 2e-2 * want.abs())).all()), f"{err.max().item():.3e}"
     new.disable()
+
+
+def test_manager_mode_decode_is_one_fused_call_and_equals_internal_mode(device):
+    """With a manager attached (the engine's ``--use-kv-manager`` mode, kv_cache.py:378-381) a decode
+    step takes the same fused append + attention call as internal mode: one library call per layer
+    and token, output and pools bit-identical to the internal-mode operator."""
+    from aicomp_amd import _lib
+    B, hq, g, d, layers = 3, 16, 4, 128, 2
+    hkv = hq // g
+    mgr = akv.KVCacheManager(num_layers=layers, max_batch_size=4, max_seq_len=128, num_heads=hq, head_dim=d,
+                             dtype=torch.bfloat16, device=device, num_kv_heads=hkv)
+    mgr.allocate(B)
+    ext = [akv.CachedScaledDotProductAttention(i, 128) for i in range(layers)]
+    own = [akv.CachedScaledDotProductAttention(i, 128, num_kv_groups=g) for i in range(layers)]
+    for a, b in zip(ext, own):
+        a.set_kv_manager(mgr); a.enable(); b.enable()
+    torch.manual_seed(5)
+    mk = lambda n, h: (torch.randn(B, h, n, d, device=device) * 0.7).to(torch.bfloat16)
+    ex = lambda x: x.repeat_interleave(g, 1)
+    lib = _lib.load()
+    calls = []
+    # every entry point that launches work (the sizing helpers are host arithmetic)
+    names = [s for s in _lib.SYMBOLS if s not in ("aicomp_kv_version", "aicomp_kv_last_error",
+                                                  "aicomp_paged_decode_workspace_bytes",
+                                                  "aicomp_paged_decode_partition_size")]
+    real = {s: getattr(lib, s) for s in names}
+
+    def counting(name):
+        def f(*a):
+            calls.append(name)
+            return real[name](*a)
+        return f
+
+    for n in (21, 1, 1, 1, 1):                       # prompt, then decode steps across a block boundary
+        for layer in range(layers):
+            q, k, v = mk(n, hq), mk(n, hkv), mk(n, hkv)
+            want = own[layer](q, ex(k), ex(v), is_causal=True)
+            del calls[:]
+            for s in names:
+                setattr(lib, s, counting(s))
+            try:
+                got = ext[layer](q, ex(k), ex(v), is_causal=True)
+            finally:
+                for s in names:
+                    setattr(lib, s, real[s])
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"n={n} layer {layer}"
+            if n == 1:
+                assert calls == ["aicomp_paged_decode_attn_append"], calls
+            else:
+                assert calls == ["aicomp_kv_append", "aicomp_paged_prefill_attn"], calls
+        assert mgr.get_seq_len() == ext[0].cache_pos == own[0].cache_pos
+    for layer in range(layers):
+        assert torch.equal(mgr._cache[layer].k_pool.view(torch.int16), own[layer].cache_k.view(torch.int16))
+        assert torch.equal(mgr._cache[layer].v_pool.view(torch.int16), own[layer].cache_v.view(torch.int16))
+    # the manager's own errors still come first (kv_cache.py:132-136, 152-156)
+    with pytest.raises(ValueError):
+        mgr.decode_step(7, mk(1, hq), mk(1, hkv), mk(1, hkv), 0, 0.1)
+    with pytest.raises(ValueError):
+        mgr.decode_step(0, mk(1, hq), mk(1, hkv), mk(1, hkv), 128, 0.1)
