@@ -28,6 +28,7 @@ Token t of a sequence lives in slot ``block_table[t // BS] * BS + t % BS``.
 """
 from __future__ import annotations
 
+import os
 from collections import deque
 from dataclasses import dataclass
 from typing import Deque, Dict, Iterable, List, Optional
@@ -39,6 +40,63 @@ import torch
 class OutOfBlocks(ValueError):
     """The pool has fewer free blocks than the request needs (the reference's cache
     overflow is a ``ValueError`` too: opt_prime/opt_prime/kv_cache.py:152-156)."""
+
+
+class PlanError(ValueError):
+    """A step plan that would make the kernels read or write outside what it owns."""
+
+
+def check_plan(plan: "StepPlan", num_blocks: int, block_size: int) -> None:
+    """Host-side self-check of a plan, from its host arrays, before anything is launched on it.
+
+    The kernels do not fault on a bad plan: an append row whose slot is outside the pool is
+    skipped and a block id outside the pool is clamped into it, so a planner bug would show up as
+    silently wrong attention.  This makes it loud: every slot inside the pool and used once, every
+    table entry a sequence needs inside the pool and owned by that sequence alone, lengths within
+    the table, chunk rows consistent with the lengths, slots and positions consistent with the table.
+    Raises ``PlanError``.
+    """
+    bt, cl, cu = plan.host_block_table, plan.host_context_lens, plan.host_cu_q_lens
+    slot, pos = plan.host_slot_mapping, plan.host_positions
+    S = len(plan.seq_ids)
+    T = int(plan.total_new_tokens)
+    if bt.shape[0] != S or cl.shape[0] != S or cu.shape[0] != S + 1 or slot.shape[0] != T or pos.shape[0] != T:
+        raise PlanError(f"plan arrays do not match {S} sequences / {T} new tokens")
+    if cu[0] != 0 or cu[-1] != T or (np.diff(cu) < 0).any():
+        raise PlanError(f"cu_q_lens is not a prefix sum ending at {T}: {cu.tolist()}")
+    new = np.diff(cu)
+    if (new != plan.new_lens).any():
+        raise PlanError("cu_q_lens and new_lens disagree")
+    if (cl < new).any() or (cl <= 0).any():
+        bad = int(np.flatnonzero((cl < new) | (cl <= 0))[0])
+        raise PlanError(f"sequence row {bad}: context length {int(cl[bad])} < its {int(new[bad])} new tokens")
+    if (cl > bt.shape[1] * block_size).any():
+        bad = int(np.flatnonzero(cl > bt.shape[1] * block_size)[0])
+        raise PlanError(f"sequence row {bad}: context length {int(cl[bad])} exceeds the table width "
+                        f"{bt.shape[1]} x {block_size}")
+    if T and ((slot < 0).any() or (slot >= num_blocks * block_size).any()):
+        bad = int(np.flatnonzero((slot < 0) | (slot >= num_blocks * block_size))[0])
+        raise PlanError(f"new token {bad}: slot {int(slot[bad])} is outside the pool of "
+                        f"{num_blocks} x {block_size} slots")
+    if T and np.unique(slot).size != T:
+        raise PlanError("two new tokens share a slot")
+    need = -(-cl.astype(np.int64) // block_size)
+    owned = []
+    for r in range(S):
+        ids = bt[r, :need[r]]
+        if ((ids < 0) | (ids >= num_blocks)).any():
+            bad = int(ids[(ids < 0) | (ids >= num_blocks)][0])
+            raise PlanError(f"sequence row {r}: block id {bad} is outside the pool of {num_blocks} blocks")
+        owned.append(ids)
+        p = pos[cu[r]:cu[r + 1]]
+        if (p != np.arange(cl[r] - new[r], cl[r])).any():
+            raise PlanError(f"sequence row {r}: positions are not {int(cl[r] - new[r])}..{int(cl[r]) - 1}")
+        if (slot[cu[r]:cu[r + 1]] != ids[p // block_size].astype(np.int64) * block_size + p % block_size).any():
+            raise PlanError(f"sequence row {r}: slots do not follow from its block table")
+    if owned:
+        allb = np.concatenate(owned)
+        if np.unique(allb).size != allb.size:
+            raise PlanError("two sequences of the plan share a block")
 
 
 class BlockAllocator:
@@ -195,7 +253,12 @@ class StepPlanner:
 
     def __init__(self, num_blocks: int, block_size: int = 16, max_seqs: int = 256,
                  max_seq_len: int = 8192, max_num_batched_tokens: int = 4096,
-                 prefill_chunk: int = 512, device="cuda", staging_depth: int = 4) -> None:
+                 prefill_chunk: int = 512, device="cuda", staging_depth: int = 4,
+                 check_plans: Optional[bool] = None) -> None:
+        # debug flag: run check_plan on every plan before its host-to-device copy (also switched on
+        # by the environment variable AICOMP_CHECK_PLANS=1); off by default, it costs host time
+        self.check_plans = (os.environ.get("AICOMP_CHECK_PLANS", "0") not in ("", "0")) if check_plans is None \
+            else bool(check_plans)
         if max_seqs <= 0 or max_seq_len <= 0 or max_num_batched_tokens <= 0 or prefill_chunk <= 0:
             raise ValueError("max_seqs, max_seq_len, max_num_batched_tokens and prefill_chunk must be positive")
         self.alloc = BlockAllocator(num_blocks, block_size)
@@ -444,6 +507,12 @@ class StepPlanner:
             slot[cu[npre]:] = bt[np.arange(npre, S), p1 // BS].astype(np.int64) * BS + p1 % BS
             posn[cu[npre]:] = p1
         np.add(start, new_lens, out=cl)
+        if self.check_plans:
+            probe = StepPlan(seq_ids=[self._id_of[int(r)] for r in rows], num_prefill_seqs=npre, new_lens=new_lens,
+                             max_q_len=0, total_new_tokens=T, block_table=None, context_lens=None, cu_q_lens=None,
+                             slot_mapping=None, positions=None, preempted=preempted, host_block_table=bt,
+                             host_context_lens=cl, host_cu_q_lens=cu, host_slot_mapping=slot, host_positions=posn)
+            check_plan(probe, self.alloc.num_blocks, BS)       # raises before anything reaches the device
         self._len[rows] = cl
         d = self._staging.upload(i, end)
         dv = d[:end]

@@ -30,6 +30,8 @@ int launch_kv_append(const void* key, const void* value, int64_t token_stride, i
 
 bool prefill_mfma_supported(const DecodeArgs& a, int max_q_len);
 int launch_prefill_mfma(const DecodeArgs& a, int max_q_len);
+bool prefill_tiled_supported(const DecodeArgs& a, int max_q_len);
+int launch_prefill_tiled(const DecodeArgs& a, int max_q_len);
 
 static int check_common(int hq, int hkv, int d, int bs, int max_blocks, int64_t num_blocks,
                         int q_dtype, int kv_dtype, const float* k_scale, const float* v_scale,
@@ -405,8 +407,11 @@ int aicomp_paged_prefill_attn(void* out, const void* query, const void* k_pool, 
     a.v_scale = kv_dtype == AICOMP_KV_FP8_E4M3 ? v_scale : nullptr;
     a.stream = (hipStream_t)stream;
     if (prefill_mfma_supported(a, max_q_len)) return launch_prefill_mfma(a, max_q_len);
-    // shapes outside the MFMA kernel: every query row as its own unsplit
-    // attention problem over its causal prefix (vector-ALU kernel)
+    // float32 models, head_dim 256, other block sizes: the tiled vector-ALU kernel (K/V staged in
+    // LDS once per 32 query rows)
+    if (prefill_tiled_supported(a, max_q_len)) return launch_prefill_tiled(a, max_q_len);
+    // what is left (pools that cannot be read 16 bytes at a time): every query row as its own
+    // unsplit attention problem over its causal prefix
     a.partition_size = (int)(((int64_t)max_blocks_per_seq * block_size + block_size - 1) /
                              block_size * block_size);
     a.num_parts = 1;

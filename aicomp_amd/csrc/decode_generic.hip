@@ -102,7 +102,8 @@ __device__ __forceinline__ void row_info(int64_t row, const int32_t* cu, const i
         seq = lo;
         int n = cu[lo + 1] - cu[lo];
         int i = (int)(row - cu[lo]);
-        len = ctx[lo] - n + i + 1;       // bottom-right aligned causal mask
+        len = ctx[lo] < n ? 0 : ctx[lo] - n + i + 1;       // bottom-right aligned causal mask; a context
+                                                            // shorter than its chunk: zero rows
     }
     if (len < 0) len = 0;
 }

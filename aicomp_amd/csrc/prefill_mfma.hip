@@ -203,7 +203,18 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     const int ctx = min(p.context_lens[seq], p.max_blocks * BS);
     const int prior = ctx - n;
     const int q0 = qtile * pos_per_wg;
-    if (q0 >= n || n <= 0 || prior < 0) return;
+    if (q0 >= n || n <= 0) return;
+    if (prior < 0) {
+        // a context shorter than the chunk itself: there is no consistent set of keys, the rows
+        // are defined as zero (the vector-ALU kernel gives the same) rather than left unwritten
+        for (int i = tid; i < 4 * WROWS * (DH / 8); i += 256) {
+            const int row = i / (DH / 8), chunk = i % (DH / 8);
+            const int pos = q0 + row / p.gpack, hd = hgroup * p.gpack + row % p.gpack;
+            if (pos < n)
+                *(uint4*)((uint16_t*)p.out + ((int64_t)(q_begin + pos) * p.hq + hd) * DH + 8 * chunk) = make_uint4(0, 0, 0, 0);
+        }
+        return;
+    }
 
     // rows of this lane's columns: row = WROWS*w + CR*c + (column, or column / 2) -> (position, head)
     const int kvh = (hgroup * p.gpack) / p.group;          // workgroup-uniform

@@ -117,7 +117,8 @@ template <typename T> __device__ __forceinline__ float f16_raw_bound(float q_sca
         const float y = (q_scaled - fmaxf(5.9604645e-8f, fabsf(q_scaled) * 9.765625e-4f)) * temperature;
         return y - fabsf(y) * 9.5367431640625e-7f;
     } else {
-        return __builtin_inff();
+        (void)q_scaled; (void)temperature;
+        return 0.f;                                    // not used for the other types
     }
 }
 template <typename T> __device__ __forceinline__ float apply_temperature(float x, float temperature);
@@ -497,7 +498,11 @@ sample_kernel(SampleParams p) {
         // prefilter on the raw float, one compare per element.  It lets through whatever the key
         // order would (plus -0.0 next to +0.0, and everything when the bound is below -inf, whose
         // key decodes to a NaN); the exact test on the scaled key follows.
-        const float raw_lo = fminf(key_value(key_lo), f16_raw_bound<T>(key_value(key_ls), temp));
+        float raw_lo = key_value(key_lo);              // may be a NaN (a bound below -inf): lets everything through
+        if constexpr (std::is_same<T, f16_t>::value) {
+            const float b = f16_raw_bound<T>(key_value(key_ls), temp);
+            if (b < raw_lo) raw_lo = b;
+        }
         for_each_logit<T>(row, 0, V, 1.f, tid, NT, vec_ok, [&](int i, float x) {
             if (!(x < raw_lo)) {
                 const uint32_t key = order_key(apply_temperature<T>(x, temp));
@@ -646,9 +651,12 @@ sample_kernel(SampleParams p) {
                 // raw prefilter: the scaled bound times the temperature, lowered by more than the division
                 // (and, for bf16 rows, the rounding of the quotient) can move a value
                 const float t_raw = key_value(key_lo_s) * temp;
-                const float raw_lo = fminf(temp == 1.f ? key_value(key_lo_s)
-                                                       : t_raw - fabsf(t_raw) * (sizeof(T) == 2 ? 0.0078125f : 9.5367431640625e-7f),
-                                           f16_raw_bound<T>(key_value(key_lo_s), temp));
+                float raw_lo = temp == 1.f ? key_value(key_lo_s)
+                                           : t_raw - fabsf(t_raw) * (sizeof(T) == 2 ? 0.0078125f : 9.5367431640625e-7f);
+                if constexpr (std::is_same<T, f16_t>::value) {
+                    const float b = f16_raw_bound<T>(key_value(key_lo_s), temp);
+                    if (b < raw_lo) raw_lo = b;
+                }
                 for_each_logit<T>(row, 0, V, 1.f, tid, NT, vec_ok, [&](int i, float x) {
                     if (!(x < raw_lo)) {
                         const uint32_t key = order_key(apply_temperature<T>(x, temp));

@@ -94,6 +94,12 @@ class ScheduleGeneration:
 
     def __init__(self, model: Callable[[torch.Tensor, torch.Tensor], torch.Tensor],
                  backend: PagedAttentionBackend, planner: StepPlanner) -> None:
+        # a token whose position has no row in the rotary tables would be left unrotated and
+        # unstored by the fused rotary + append launch: refuse the combination up front
+        cos = getattr(backend, "cos", None)
+        if cos is not None and planner.max_seq_len > cos.shape[0]:
+            raise ValueError(f"the planner admits sequences of {planner.max_seq_len} tokens but the backend's "
+                             f"rotary tables hold {cos.shape[0]} positions (max_positions)")
         self.model = model
         self.backend = backend
         self.planner = planner

@@ -203,7 +203,8 @@ int aicomp_paged_decode_partition_size(int batch, int num_q_heads, int num_kv_he
  * The chunk's own K/V rows must already be in the pool (append first).
  *
  *   out, query     [T, Hq, D] of q_dtype, rows of sequence s are cu_q_lens[s]..cu_q_lens[s+1]
- *   context_lens   [S] int32: prior context + chunk length
+ *   context_lens   [S] int32: prior context + chunk length; a sequence whose length is
+ *                  smaller than its chunk gets zero output rows (no error)
  *   cu_q_lens      [S+1] int32 prefix sums of the chunk lengths
  *   max_q_len      host-side upper bound of the chunk lengths (sizes the grid)
  * Mask: query i of a chunk with prior context P sees keys j <= P + i

@@ -151,7 +151,7 @@ class Sim:
 
 
 def test_planner_prefill_then_decode_matches_oracle():
-    p = StepPlanner(num_blocks=64, max_seqs=8, max_seq_len=256, max_num_batched_tokens=64,
+    p = StepPlanner(check_plans=True, num_blocks=64, max_seqs=8, max_seq_len=256, max_num_batched_tokens=64,
                     prefill_chunk=24, device="cpu")
     sim = Sim(p)
     p.add_request("a", 50, 10)
@@ -223,7 +223,7 @@ def test_planner_max_seq_len_overflow_raises():
 
 
 def test_planner_token_budget_and_max_seqs():
-    p = StepPlanner(num_blocks=256, max_seqs=3, max_seq_len=512, max_num_batched_tokens=40,
+    p = StepPlanner(check_plans=True, num_blocks=256, max_seqs=3, max_seq_len=512, max_num_batched_tokens=40,
                     prefill_chunk=32, device="cpu")
     sim = Sim(p)
     for i in range(5):
@@ -241,7 +241,7 @@ def test_planner_token_budget_and_max_seqs():
 
 def test_planner_preemption_recomputes_and_everything_finishes():
     # 12 blocks = 192 tokens of pool for sequences that want up to 80 each: evictions are certain
-    p = StepPlanner(num_blocks=12, max_seqs=6, max_seq_len=96, max_num_batched_tokens=64,
+    p = StepPlanner(check_plans=True, num_blocks=12, max_seqs=6, max_seq_len=96, max_num_batched_tokens=64,
                     prefill_chunk=32, device="cpu")
     sim = Sim(p, seed=3)
     want = {}
@@ -277,7 +277,7 @@ def test_planner_oldest_cannot_be_preempted_raises_when_alone():
 
 
 def test_planner_random_soak_against_oracle():
-    p = StepPlanner(num_blocks=48, max_seqs=10, max_seq_len=160, max_num_batched_tokens=96,
+    p = StepPlanner(check_plans=True, num_blocks=48, max_seqs=10, max_seq_len=160, max_num_batched_tokens=96,
                     prefill_chunk=40, device="cpu", staging_depth=2)
     sim = Sim(p, seed=7)
     nxt = 0
@@ -298,3 +298,51 @@ def test_planner_random_soak_against_oracle():
         if plan is not None:
             sim.apply(plan)
     assert nxt > 50
+
+
+def test_check_plan_catches_corrupted_plans():
+    """The kernels skip or clamp what lies outside the pool instead of faulting, so a planner bug
+    would be silent: the host-side self-check names it before the plan reaches the device."""
+    import copy
+    from aicomp_amd.block_manager import PlanError, check_plan
+    pl = StepPlanner(num_blocks=64, max_seqs=8, max_seq_len=256, max_num_batched_tokens=512, prefill_chunk=64,
+                     device="cpu", check_plans=True)
+    for i, n in enumerate((40, 70, 5)):
+        pl.add_request(i, n)
+    plan = pl.schedule()                       # passes its own check
+    check_plan(plan, 64, 16)
+
+    def broken(**edit):
+        p = copy.copy(plan)
+        for k, fn in edit.items():
+            a = getattr(plan, k).copy()
+            fn(a)
+            setattr(p, k, a)
+        return p
+
+    def slot_out(a): a[3] = 64 * 16 + 5
+    def slot_neg(a): a[0] = -1
+    def slot_dup(a): a[1] = a[0]
+    def block_out(a): a[1, 0] = 64
+    def block_shared(a): a[2, 0] = a[0, 0]
+    def ctx_long(a): a[0] = 256 + 16 * 2
+    def ctx_short(a): a[1] = 3
+    def pos_wrong(a): a[2] += 1
+    for edit in (dict(host_slot_mapping=slot_out), dict(host_slot_mapping=slot_neg), dict(host_slot_mapping=slot_dup),
+                 dict(host_block_table=block_out), dict(host_block_table=block_shared),
+                 dict(host_context_lens=ctx_long), dict(host_context_lens=ctx_short), dict(host_positions=pos_wrong)):
+        with pytest.raises(PlanError):
+            check_plan(broken(**edit), 64, 16)
+    # inside the planner: a corrupted table row is caught by schedule() itself, before the upload
+    r = pl._row_of[1]
+    pl._tab[r, 0] = 99
+    with pytest.raises(PlanError):
+        pl.schedule()
+
+
+def test_check_plan_flag_defaults_to_the_environment(monkeypatch):
+    monkeypatch.delenv("AICOMP_CHECK_PLANS", raising=False)
+    assert StepPlanner(num_blocks=8, device="cpu").check_plans is False
+    monkeypatch.setenv("AICOMP_CHECK_PLANS", "1")
+    assert StepPlanner(num_blocks=8, device="cpu").check_plans is True
+    assert StepPlanner(num_blocks=8, device="cpu", check_plans=False).check_plans is False

@@ -69,3 +69,17 @@ def test_clear_cache_releases_blocks_and_prefill_restarts():
     assert planner.alloc.num_used == 0 and not planner.has_work()
     out = gen.prefill(torch.ones(1, 4, dtype=torch.long))
     assert out.tolist() == [[1.0, 3.0]]
+
+
+def test_rotary_tables_must_cover_the_planner_lengths():
+    """A token beyond the rotary tables would be neither rotated nor stored by the fused launch:
+    the driver refuses a planner that admits longer sequences than the backend's tables hold."""
+    planner = StepPlanner(num_blocks=64, max_seqs=8, max_seq_len=128, device="cpu")
+
+    class RopeBackend(EchoBackend):
+        cos = torch.zeros(64, 16)
+
+    with pytest.raises(ValueError, match="rotary tables hold 64"):
+        ScheduleGeneration(lambda ids, pos: ids, RopeBackend(), planner)
+    RopeBackend.cos = torch.zeros(128, 16)
+    ScheduleGeneration(lambda ids, pos: ids, RopeBackend(), planner)

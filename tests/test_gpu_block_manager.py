@@ -21,7 +21,7 @@ BF16_ATOL, BF16_RTOL = 1e-2, 2e-2
 def run_serving(device, kv_dtype, steps, seed, num_blocks=96, hq=8, hkv=2, d=128):
     g = torch.Generator().manual_seed(seed)
     rng = np.random.default_rng(seed)
-    p = StepPlanner(num_blocks=num_blocks, max_seqs=12, max_seq_len=400, max_num_batched_tokens=256,
+    p = StepPlanner(check_plans=True, num_blocks=num_blocks, max_seqs=12, max_seq_len=400, max_num_batched_tokens=256,
                     prefill_chunk=96, device=device)
     fp8 = kv_dtype == torch.float8_e4m3fn
     # pools start non-finite: nothing beyond a context may leak into a result

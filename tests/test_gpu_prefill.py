@@ -142,6 +142,33 @@ def test_prefill_fp32_and_other_shapes_use_the_generic_kernel(device):
     assert np.abs(got - oracle(c)).max() <= 1e-5
 
 
+@pytest.mark.parametrize("hq,hkv,d,bs", [(8, 2, 128, 16), (4, 4, 64, 16), (6, 2, 128, 16), (16, 2, 64, 32),
+                                         (4, 1, 256, 16)])
+def test_prefill_fp32_tiled_kernel(device, hq, hkv, d, bs):
+    """float32 models (the reference's ``--dtype float32``) take the tiled vector kernel: a fresh
+    512-token prompt, a continuation across tile and block boundaries, ragged and one-token chunks,
+    groups of 1, 3 (one head per workgroup), 4 and 8; <= 1e-5 against the float64 oracle."""
+    c = build_case(device, priors=[0, 300, 5, 0, 63, 31], news=[512, 130, 33, 1, 1, 70], hq=hq, hkv=hkv, d=d, bs=bs,
+                   dtype=torch.float32, seed=d + bs)
+    got = run(c, max_q_len=512)
+    assert torch.isfinite(got).all()
+    assert np.abs(to_f64(got) - oracle(c)).max() <= 1e-5
+
+
+@pytest.mark.parametrize("dtype,kv_dtype,d,bs", [(torch.bfloat16, None, 256, 16), (torch.bfloat16, None, 128, 32),
+                                                 (torch.float16, None, 256, 16),
+                                                 (torch.bfloat16, torch.float8_e4m3fn, 256, 16),
+                                                 (torch.float16, torch.float8_e4m3fn, 128, 8)])
+def test_prefill_16bit_shapes_outside_the_matrix_core_kernel(device, dtype, kv_dtype, d, bs):
+    """head_dim 256 and block sizes other than 16 with 16-bit queries: the tiled kernel widens the pool
+    rows to float32 in LDS; NaN / Inf beyond every context must not reach the output."""
+    c = build_case(device, priors=[0, 200, 37], news=[300, 64, 17], hq=8, hkv=2, d=d, bs=bs, dtype=dtype,
+                   kv_dtype=kv_dtype, seed=3)
+    got = run(c, max_q_len=300)
+    assert torch.isfinite(got.float()).all()
+    assert_close_attn(to_f64(got), oracle(c), BF16_ATOL, BF16_RTOL, f"tiled {dtype} D {d} BS {bs}")
+
+
 def test_prefill_fp8_kv(device):
     c = build_case(device, priors=[0, 100], news=[64, 40], hq=16, hkv=2, d=128, kv_dtype=torch.float8_e4m3fn)
     got = to_f64(run(c))
@@ -207,3 +234,20 @@ def test_prefill_head_dim_64_long_chunks(device):
     want = torch.nn.functional.scaled_dot_product_attention(
         q, k.repeat_interleave(4, 0)[None], v.repeat_interleave(4, 0)[None], is_causal=True)
     assert_close_attn(got[:L], want[0].permute(1, 0, 2).double().numpy(), BF16_ATOL, BF16_RTOL, "causal D64")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_prefill_context_shorter_than_chunk_gives_zero_rows(device, dtype):
+    """A sequence whose context length is smaller than its chunk (an inconsistent plan) must not
+    leave its output rows unwritten: both kernels define them as zero, the other chunks are unaffected."""
+    c = build_case(device, priors=[10, 0, 33], news=[130, 140, 20], hq=8, hkv=2, d=128, dtype=dtype, poison=False)
+    want = oracle(c)
+    ctx = c["ctx"].clone()
+    ctx[1] = 100                                   # 140 new rows, but only 100 tokens of context
+    c2 = dict(c, ctx=ctx)
+    got = run(c2, max_q_len=140)
+    lo, hi = int(c["cu"][1]), int(c["cu"][2])
+    assert float(got[lo:hi].float().abs().max()) == 0.0
+    keep = np.r_[0:lo, hi:got.shape[0]]
+    tol = (BF16_ATOL, BF16_RTOL) if dtype == torch.bfloat16 else (1e-5, 0.0)
+    assert_close_attn(to_f64(got)[keep], want[keep], tol[0], tol[1], "chunks beside the inconsistent one")
