@@ -25,9 +25,20 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 METRIC = "decode-attn HBM GB/s (% peak) + tokens/s, Llama-3-8B paged KV, 1 GPU"
 
-# HBM bytes per decode launch of the Llama-3-8B shape from rocprofv3 --pmc
-# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, the factors a 1 GiB device copy gives), main + merge kernel.
-MEASURED_TRAFFIC_BYTES = 651.3e6   # profiles/decode_llama3_8b_decode.md
+
+
+def measured_traffic_bytes():
+    """HBM bytes per decode call of the Llama-3-8B shape as the kept rocprofv3 counter summary gives
+    them (--pmc FETCH_SIZE / WRITE_SIZE, scaled by what a 1 GiB device copy reads on the same
+    counters; main + merge kernel): read from profiles/decode_llama3_8b_decode.md so that the figure
+    in the JSON line and the summary cannot drift apart.  None if the summary is missing."""
+    import re
+    try:
+        with open(os.path.join(ROOT, "profiles", "decode_llama3_8b_decode.md")) as f:
+            m = re.search(r"Total HBM traffic per call:\s*([0-9.]+)\s*MB", f.read())
+        return float(m.group(1)) * 1e6 if m else None
+    except OSError:
+        return None
 
 
 def _events(n):
@@ -183,10 +194,22 @@ def run_decode_config(name, steps, warmup, dev):
                                                     qd.dtype, w.k_pool.dtype),
         "kv_dtype": str(w.k_pool.dtype).replace("torch.", ""),
     }
+    mfma_shape = (w.shape.head_dim in (64, 128) and w.shape.block_size == 16 and qd.dtype in (torch.bfloat16, torch.float16))
+    balanced = mfma_shape and w.shape.head_dim == 128 and (S - npre) <= 1024
+    res["roofline"] = {
+        "kernel": ("streamk_decode_kernel + streamk_reduce_kernel" if balanced else
+                   "paged_decode_mfma_kernel + split_reduce_kernel" if mfma_shape else
+                   "paged_attn_generic_kernel + split_reduce_kernel"),
+        "bound": "hbm", "achieved": res["decode_GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": res["decode_frac_hbm_peak"], "algorithmic_bytes": res["decode_bytes"], "avg_launch_us": res["decode_us"]}
     if npre:
         res.update({"prefill_us": t_pre * 1e6, "prefill_flops": w.prefill_flops(),
                     "prefill_TFLOPs": w.prefill_flops() / t_pre / 1e12,
                     "prefill_frac_mfma_peak": w.prefill_flops() / t_pre / 1e12 / MFMA_BF16_PEAK_TFLOPS})
+        res["prefill_roofline"] = {
+            "kernel": "paged_prefill_mfma_kernel", "bound": "mfma", "achieved": res["prefill_TFLOPs"],
+            "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": res["prefill_frac_mfma_peak"],
+            "algorithmic_flop": res["prefill_flops"], "avg_launch_us": res["prefill_us"]}
     return res, w
 
 
@@ -261,17 +284,24 @@ def sampler_bench(dev, batch=64, vocab=128256, temperature=0.8, top_k=50, top_p=
     return res
 
 
-def prefill_shapes_bench(dev, reps=5):
-    """The chunked-prefill kernel on shapes with many more workgroups than the named mixed step
+def prefill_shapes_bench(dev, reps=20):
+    """The chunked-prefill kernels on shapes with many more workgroups than the named mixed step
     (512 workgroups there, two per CU, bounded by the longest of them): fresh long prompts and a
-    batch of chunks with prior context.  Synthetic bf16 K/V, 32/8 heads, D 128."""
+    batch of chunks with prior context.  Synthetic K/V, 32/8 heads.  Every shape is first run for
+    about 30 ms untimed (the clock of an idle GPU takes that long to settle: the first launches after
+    a pause run 10-15 % slower), then `reps` launches are timed between two events."""
     import math
     import torch
     from aicomp_amd import ops
     hq, hkv = 32, 8
     out = []
-    for nseq, n, prior, d, fp8 in ((1, 8192, 0, 128, False), (4, 4096, 0, 128, False), (16, 512, 2048, 128, False),
-                                   (16, 512, 2048, 128, True), (16, 512, 2048, 64, False)):
+    for nseq, n, prior, d, kvt, qt in ((1, 8192, 0, 128, torch.bfloat16, torch.bfloat16),
+                                       (4, 4096, 0, 128, torch.bfloat16, torch.bfloat16),
+                                       (16, 512, 2048, 128, torch.bfloat16, torch.bfloat16),
+                                       (16, 512, 2048, 128, torch.float8_e4m3fn, torch.bfloat16),
+                                       (16, 512, 2048, 64, torch.bfloat16, torch.bfloat16),
+                                       (16, 512, 2048, 128, torch.float16, torch.float16),
+                                       (1, 2048, 0, 128, torch.float32, torch.float32)):
         ctx = prior + n
         nblk = math.ceil(ctx / 16)
         nb = nseq * nblk + 1
@@ -280,21 +310,26 @@ def prefill_shapes_bench(dev, reps=5):
         k = torch.randn(nb, hkv, 16, d, device=dev) * 0.5
         v = torch.randn(nb, hkv, 16, d, device=dev) * 0.5
         ks = vs = None
-        if fp8:
+        if kvt == torch.float8_e4m3fn:
             ks = (k.abs().amax(dim=(0, 2, 3)) / 448).float().contiguous()
             vs = (v.abs().amax(dim=(0, 2, 3)) / 448).float().contiguous()
-            k = (k / ks[None, :, None, None]).to(torch.float8_e4m3fn)
-            v = (v / vs[None, :, None, None]).to(torch.float8_e4m3fn)
+            k = (k / ks[None, :, None, None]).to(kvt)
+            v = (v / vs[None, :, None, None]).to(kvt)
         else:
-            k, v = k.to(torch.bfloat16), v.to(torch.bfloat16)
-        q = torch.randn(nseq * n, hq, d, device=dev).to(torch.bfloat16)
+            k, v = k.to(kvt), v.to(kvt)
+        q = torch.randn(nseq * n, hq, d, device=dev).to(qt)
         o = torch.empty_like(q)
         cl = torch.full((nseq,), ctx, dtype=torch.int32, device=dev)
         cu = (torch.arange(nseq + 1, dtype=torch.int32) * n).to(dev)
         call = lambda: ops.paged_prefill_attn(o, q, k, v, table, cl, cu, 1 / math.sqrt(d), max_q_len=n,
                                               k_scale=ks, v_scale=vs)
-        for _ in range(2):
-            call()
+        call()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 0.03:
+            for _ in range(4):
+                call()
+            torch.cuda.synchronize()
         e0, e1 = _events(2)
         e0.record()
         for _ in range(reps):
@@ -303,10 +338,14 @@ def prefill_shapes_bench(dev, reps=5):
         torch.cuda.synchronize()
         t = e0.elapsed_time(e1) / reps * 1e-3
         flops = nseq * 4 * hq * d * (n * prior + n * (n + 1) / 2)
+        f32 = qt == torch.float32
+        peak = 157.3 if f32 else MFMA_BF16_PEAK_TFLOPS          # fp32 vector / matrix peak, published
+        name = lambda t_: str(t_).replace("torch.", "")
         out.append({"chunks": nseq, "new_tokens": n, "prior": prior, "head_dim": d,
-                    "kv_dtype": "float8_e4m3fn" if fp8 else "bfloat16", "us": round(t * 1e6, 1),
+                    "q_dtype": name(qt), "kv_dtype": name(kvt), "us": round(t * 1e6, 1),
                     "TFLOPs": round(flops / t / 1e12, 1),
-                    "frac_mfma_peak": round(flops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
+                    "kernel": "paged_prefill_tiled_kernel" if f32 else "paged_prefill_mfma_kernel",
+                    "peak_TFLOPs": peak, "frac_mfma_peak": round(flops / t / 1e12 / peak, 4)})
         del k, v, q, o
         torch.cuda.empty_cache()
     return out
@@ -413,7 +452,7 @@ def cpu_baseline(w, budget_s=20.0):
     ks = None if w.k_scale is None else w.k_scale.cpu()
     vs = None if w.v_scale is None else w.v_scale.cpu()
     B = q.shape[0]
-    n = min(B, 8)
+    n = min(B, 4 if budget_s < 10 else 8)
 
     def run(nseq):
         t0 = time.perf_counter()
@@ -496,7 +535,7 @@ def main():
         "roofline": {"kernel": "streamk_decode_kernel<bf16> (append fused) + streamk_reduce_kernel (one decode call)",
                      "bound": "hbm", "achieved": main_res["decode_GBs"], "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": main_res["decode_GBs"] / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES,
+                     "traffic": measured_traffic_bytes(),
                      "algorithmic_bytes": main_res["decode_bytes"],
                      "avg_launch_us": main_res["decode_us"]},
         "append": {"us": main_res["append_us"], "GB/s": main_res["append_GBs"],
@@ -518,9 +557,15 @@ def main():
         for name in ("decode_fp32_small", "long_context_skewed", "chunked_prefill_mixed",
                      "llama3_70b_decode_fp8", "llama32_1b_decode"):
             r, ww = run_decode_config(name, args.steps, args.warmup, dev)
+            if not args.no_cpu:
+                # the reference's CPU path on the same batch, in the workload's own dtype (fp32 for
+                # the small anchor shape, which is defined on that path); a few seconds each
+                r["cpu_baseline"] = cpu_baseline(ww, budget_s=5.0)
             del ww
             torch.cuda.empty_cache()
-            extra.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})
+            rnd = lambda v: round(v, 4) if isinstance(v, float) else v
+            extra.append({k: ({kk: rnd(vv) for kk, vv in v.items()} if isinstance(v, dict) else rnd(v))
+                          for k, v in r.items()})
         line["other_workloads"] = extra
     print(json.dumps(line))
 
