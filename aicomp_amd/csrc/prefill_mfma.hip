@@ -29,8 +29,9 @@
 // head_dim     128 or 64, one instantiation each.
 // Per wave     16 or 32 rows (one or two column groups).  S^T = K Q^T with K rows as
 //              the A operand and the wave's query rows as B columns
-//              (v_mfma_f32_16x16x32_bf16 / _f16); online softmax per column on the raw
-//              scores with a lazily moved max: the exponentials are taken against the current
+//              (v_mfma_f32_16x16x32_bf16 / _f16), the score multiplier folded into Q and the
+//              running max into the accumulators' starting value; online softmax per column
+//              with a lazily moved max: the exponentials are taken against the current
 //              max and their sum tells whether it has to move (then, rarely, the row max is
 //              found with two lane swaps and the exponentials are redone); O^T += V^T P^T
 //              with the V^T operand read out of the row-major V tile by gfx950's transposing
@@ -243,25 +244,33 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         for (int s = 0; s < NSL; ++s)                           // k-slot s, k-group g4: elements 32s + 8*g4 ..
             qf[c][s] = *(const uint4*)(qrow + 32 * s + 8 * g4);
     }
-    // log2(e) * scale * k_scale.  The softmax below tracks the max of the raw scores, which needs
-    // a positive multiplier: a negative one (a negative k_scale) moves its sign into Q.
-    float cmul = p.qk_mul * (FP8 ? p.k_scale[kvh] : 1.f);
-    if (cmul < 0.f) {
-        cmul = -cmul;
+    // The score multiplier log2(e) * scale (* k_scale for an fp8 pool) goes into Q once, here, so
+    // that the matrix cores deliver the scores already in the exponent's units and the softmax
+    // spends no multiply on them (one rounding of q * multiplier to the 16-bit format: a relative
+    // 2^-9 per element for bf16, far below the rounding of the probabilities themselves).
+    {
+        const float cmul = p.qk_mul * (FP8 ? p.k_scale[kvh] : 1.f);
 #pragma unroll
         for (int c = 0; c < R; ++c)
 #pragma unroll
             for (int s = 0; s < NSL; ++s) {
-                uint4& u = qf[c][s];
-                u.x ^= E::SIGN_PAIR; u.y ^= E::SIGN_PAIR; u.z ^= E::SIGN_PAIR; u.w ^= E::SIGN_PAIR;
+                uint32_t* w = (uint32_t*)&qf[c][s];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    w[i] = E::pack(E::to_f32((uint16_t)(w[i] & 0xffffu)) * cmul, E::to_f32((uint16_t)(w[i] >> 16)) * cmul);
             }
     }
 
-    float m[R], lsum[R], bias[R];                // bias = -m * cmul, kept beside m
+    // m = reference max of a row in the exponent's units; its negative is what the score
+    // accumulators start from (the C operand of the first QK^T MFMA), so a score comes out of the
+    // matrix core as s - m, ready for the exponential.  The first tile starts from 0 and always
+    // takes the path that adopts the tile's own row maximum.
+    float m[R], lsum[R];
+    f32x4_t binit[R];
     f32x4_t O[R][NJ];
 #pragma unroll
     for (int c = 0; c < R; ++c) {
-        m[c] = NEG_BIG; lsum[c] = 0.f; bias[c] = -NEG_BIG * cmul;
+        m[c] = 0.f; lsum[c] = 0.f; binit[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < NJ; ++j) O[c][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
@@ -344,24 +353,44 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     // Direct-to-LDS fetch of tile t: wave w brings in block w of the tile (16 token rows) with
     // 1 KB instructions, four rows of 256 bytes or eight of 128 each; lane l of instruction q lands
     // at row RPI*q + l/CPR, chunk slot l%CPR, and the slot holds chunk (l%CPR) ^ swz(row) (the XOR
-    // swizzle that keeps the operand reads free of bank conflicts without padding), so the lane
+    // swizzle that lets the operand reads run at the full LDS rate without padding), so the lane
     // reads that chunk from the pool.  One block per wave: one table entry, one base address and
     // one LDS base per pool; the instruction's immediate offset moves the pool and the LDS address
     // together by 1 KB per q.
     static_assert(!DMA || NB == 4, "one block of the tile per wave");
     constexpr int RPI = 1024 / KROW;           // token rows one 1 KB instruction lands (4 or 8)
     constexpr int NQ = 16 / RPI;               // instructions per block and pool (4 or 2)
-    // chunk slot s of LDS row r holds chunk s ^ swz(r): sixteen consecutive rows put one chunk
-    // index into sixteen different 16-byte bank groups (256-byte rows: 16 slots; 128-byte rows:
-    // 8 slots x the two halves of the banks that even and odd rows fall into)
-    auto swz = [](int row) { return DH == 128 ? (row & 15) : ((row >> 1) & 7); };
+    // Chunk slot s of LDS row r holds chunk s ^ swz(r), with one swizzle for the K tile and one for
+    // the V tile, each fitted to how the LDS serves its operand read.  Measured on this part (a
+    // wave of reads per instruction, 16 waves): the 64 banks deliver 256 bytes per clock only when
+    // (a) every four consecutive lanes of a 16-byte read (eight of the 8-byte transposing read)
+    // address one aligned 64-byte segment, and (b) each half-wave spreads its segments evenly over
+    // the four segments of a bank line; a pattern that is merely free of bank collisions among the
+    // sixteen lanes of an MFMA row group (row-index XOR, or padded rows) runs at half that rate.
+    // K operand: lanes 4i .. 4i+3 read rows i, 4+i, 8+i, 12+i of a 16-row group at one chunk
+    // index: the row's position among those four goes into the slot's low bits, i picks the segment.
+    // V operand (transposing read): lanes 0-3 / 4-7 of a group read 32 bytes of rows g, 4+g, the
+    // next eight lanes of rows 8+g, 12+g: adjacent 32-byte units for the first pair and the second,
+    // the other half of the bank line for odd g.  With 128-byte rows (head_dim 64) even and odd
+    // rows are the two halves of a bank line by themselves.
+    auto swz_k = [](int row) {
+        const int a = (row >> 2) & 3, b = row & 3;
+        return DH == 128 ? (a | (b << 2)) : (a | ((b >> 1) << 2));
+    };
+    auto swz_v = [](int row) {
+        const int a = (row >> 2) & 3, b = row & 3;
+        return DH == 128 ? ((a | ((b & 1) << 2)) << 1) : (a << 1);
+    };
     const uint32_t dma_blk_stride = (uint32_t)p.hkv * (BS * DH * 2);              // bytes per block, < 2^32
     const char* dma_kp = (const char*)p.k_pool + (int64_t)kvh * (BS * DH * 2);   // this KV head's slice of block 0
     const char* dma_vp = (const char*)p.v_pool + (int64_t)kvh * (BS * DH * 2);
     const int dma_lrow = lane / CPR, dma_slot = lane % CPR;     // this lane's row and slot within 1 KB
-    uint32_t dma_off[NQ];                      // pool offset of this lane's chunk, less the immediate
+    uint32_t dma_offk[NQ], dma_offv[NQ];       // pool offset of this lane's chunk, less the immediate
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) dma_off[q] = dma_lrow * KROW + ((dma_slot ^ swz(RPI * q + dma_lrow)) << 4);
+    for (int q = 0; q < NQ; ++q) {
+        dma_offk[q] = dma_lrow * KROW + ((dma_slot ^ swz_k(RPI * q + dma_lrow)) << 4);
+        dma_offv[q] = dma_lrow * KROW + ((dma_slot ^ swz_v(RPI * q + dma_lrow)) << 4);
+    }
     auto fetch_dma = [&](int t, unsigned char* kb, unsigned char* vb) {
         const int first = NB * t;
         const bool tail = (t + 1) * KT > ctx || first + NB > p.max_blocks;     // workgroup-uniform
@@ -371,15 +400,17 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             // The offset is an immediate: explicit instances.  The lane offsets are made opaque once
             // per step, so that each address stays a uniform 64-bit base plus a 32-bit lane offset
             // (the load's scalar-base form) instead of a per-lane 64-bit pointer built with VALU adds.
-            uint32_t o[4] = {dma_off[0], dma_off[1], dma_off[NQ > 2 ? 2 : 0], dma_off[NQ > 2 ? 3 : 1]};
-            asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]));
+            uint32_t ok[4] = {dma_offk[0], dma_offk[1], dma_offk[NQ > 2 ? 2 : 0], dma_offk[NQ > 2 ? 3 : 1]};
+            uint32_t ov[4] = {dma_offv[0], dma_offv[1], dma_offv[NQ > 2 ? 2 : 0], dma_offv[NQ > 2 ? 3 : 1]};
+            asm volatile("" : "+v"(ok[0]), "+v"(ok[1]), "+v"(ok[2]), "+v"(ok[3]));
+            asm volatile("" : "+v"(ov[0]), "+v"(ov[1]), "+v"(ov[2]), "+v"(ov[3]));
             const char* kaddr = dma_kp + base;
             const char* vaddr = dma_vp + base;
-#define AICOMP_DMA_ROWS(addr, buf, q)                                                                               \
+#define AICOMP_DMA_ROWS(addr, o, buf, q)                                                                            \
             if constexpr (q < NQ)                                                                                   \
                 __builtin_amdgcn_global_load_lds(GLOBAL_PTR(addr + o[q]), LDS_PTR(buf + 16 * w * KROW), 16, 1024 * q, 0);
-            AICOMP_DMA_ROWS(kaddr, kb, 0) AICOMP_DMA_ROWS(kaddr, kb, 1) AICOMP_DMA_ROWS(kaddr, kb, 2) AICOMP_DMA_ROWS(kaddr, kb, 3)
-            AICOMP_DMA_ROWS(vaddr, vb, 0) AICOMP_DMA_ROWS(vaddr, vb, 1) AICOMP_DMA_ROWS(vaddr, vb, 2) AICOMP_DMA_ROWS(vaddr, vb, 3)
+            AICOMP_DMA_ROWS(kaddr, ok, kb, 0) AICOMP_DMA_ROWS(kaddr, ok, kb, 1) AICOMP_DMA_ROWS(kaddr, ok, kb, 2) AICOMP_DMA_ROWS(kaddr, ok, kb, 3)
+            AICOMP_DMA_ROWS(vaddr, ov, vb, 0) AICOMP_DMA_ROWS(vaddr, ov, vb, 1) AICOMP_DMA_ROWS(vaddr, ov, vb, 2) AICOMP_DMA_ROWS(vaddr, ov, vb, 3)
 #undef AICOMP_DMA_ROWS
         } else {
             // rows at or beyond the context take the last valid row instead (finite data for
@@ -392,9 +423,10 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             for (int q = 0; q < NQ; ++q) {
                 const int row = RPI * q + dma_lrow;
                 const int tok = min(16 * (first + w) + row, last);
-                const uint32_t off = (tok - 16 * bi) * KROW + ((dma_slot ^ swz(row)) << 4);
-                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(dma_kp + base + off), LDS_PTR(kb + (16 * w + RPI * q) * KROW), 16, 0, 0);
-                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(dma_vp + base + off), LDS_PTR(vb + (16 * w + RPI * q) * KROW), 16, 0, 0);
+                const uint32_t offk = (tok - 16 * bi) * KROW + ((dma_slot ^ swz_k(row)) << 4);
+                const uint32_t offv = (tok - 16 * bi) * KROW + ((dma_slot ^ swz_v(row)) << 4);
+                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(dma_kp + base + offk), LDS_PTR(kb + (16 * w + RPI * q) * KROW), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(dma_vp + base + offv), LDS_PTR(vb + (16 * w + RPI * q) * KROW), 16, 0, 0);
             }
         }
     };
@@ -426,14 +458,14 @@ paged_prefill_mfma_kernel(PrefillParams p) {
 #pragma unroll
         for (int h = 0; h < NH; ++h)
 #pragma unroll
-            for (int c = 0; c < R; ++c) sa[h][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            for (int c = 0; c < R; ++c) sa[h][c] = binit[c];
 #pragma unroll
         for (int s = 0; s < NSL; ++s) {
             uint4 a[NH];
 #pragma unroll
             for (int h = 0; h < NH; ++h)
-                if constexpr (DMA)   // chunk 4s + g4 of row 16h + prow sits at chunk slot (4s + g4) ^ swz(prow)
-                    a[h] = *(const uint4*)(kb + 16 * h * KROW + prow * KROW + (((4 * s + g4) ^ swz(prow)) << 4));
+                if constexpr (DMA)   // chunk 4s + g4 of row 16h + prow sits at chunk slot (4s + g4) ^ swz_k(prow)
+                    a[h] = *(const uint4*)(kb + 16 * h * KROW + prow * KROW + (((4 * s + g4) ^ swz_k(prow)) << 4));
                 else
                     a[h] = *(const uint4*)(kb + 16 * h * KROW + rd_k + s * 64);
 #pragma unroll
@@ -442,11 +474,12 @@ paged_prefill_mfma_kernel(PrefillParams p) {
                 for (int c = 0; c < R; ++c)
                     sa[h][c] = E::mfma(a[h], qf[c][s], sa[h][c]);
         }
-        // Online softmax on the raw scores: the score multiplier is folded into the exponent's
-        // fused multiply-add and the running max stays in raw units.  The max is moved lazily:
-        // the exponentials are first taken against the current max, and as long as a lane's sum of
-        // them stays <= 2^8 every P is at most 256, exact enough in bf16 and f32, and neither the
-        // max nor the accumulators are touched.  Only tiles that cross the diagonal pay for the mask.
+        // Online softmax: the scores arrive as s - m in the exponent's units (multiplier in Q, -m in
+        // the accumulators' starting value), so a probability is one exponential.  The max is moved
+        // lazily: the exponentials are first taken against the current max, and as long as a lane's
+        // sum of them stays <= 2^8 every P is at most 256, exact enough in the 16-bit format and
+        // f32, and neither the max nor the accumulators are touched.  Only tiles that cross the
+        // diagonal pay for the mask.
         const bool need_mask = sub_start + TT - 1 > wave_kv_min;       // wave-uniform
         uint4 pf[R][NH / 2];
         float alpha[R];
@@ -477,8 +510,8 @@ paged_prefill_mfma_kernel(PrefillParams p) {
                     psum = 0.f;
 #pragma unroll
                     for (int k = 0; k < NS; k += 2) {
-                        float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[k], cmul, bias[c]));
-                        float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[k + 1], cmul, bias[c]));
+                        float p0 = __builtin_amdgcn_exp2f(sc[k]);
+                        float p1 = __builtin_amdgcn_exp2f(sc[k + 1]);
                         if (MASK && dead[k]) p0 = 0.f;
                         if (MASK && dead[k + 1]) p1 = 0.f;
                         pk[k >> 1] = E::pack(p0, p1);
@@ -489,7 +522,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
                 // A row's scores sit in four lanes (l, l^16, l^32, l^48), which must share one
                 // reference max, so the whole wave takes the slow path together: row max over the
                 // lanes, rescale factor, exponentials again (the accumulator rescale is below).
-                grew[c] = __any(!(psum <= 256.f));
+                grew[c] = t == 0 || __any(!(psum <= 256.f));
                 if (grew[c]) {
                     float mx_lane = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
                                           fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
@@ -498,11 +531,14 @@ paged_prefill_mfma_kernel(PrefillParams p) {
                                                        fmaxf(fmaxf(sc[12], sc[13]), fmaxf(sc[14], sc[15]))));
                     float mx = xor16_max(mx_lane);
                     mx = xor32_max(mx);
-                    const bool up = mx > m[c];
-                    alpha[c] = up ? __builtin_amdgcn_exp2f((m[c] - mx) * cmul) : 1.f;
-                    m[c] = up ? mx : m[c];
-                    bias[c] = -m[c] * cmul;
+                    // mx is relative to the current reference; the first tile adopts it whatever its sign
+                    const float shift = (t == 0 || mx > 0.f) ? mx : 0.f;
+                    alpha[c] = t == 0 ? 0.f : __builtin_amdgcn_exp2f(-shift);
+                    m[c] += shift;
+                    binit[c] = f32x4_t{-m[c], -m[c], -m[c], -m[c]};
                     lsum[c] *= alpha[c];
+#pragma unroll
+                    for (int k = 0; k < NS; ++k) sc[k] -= shift;
                     exps();
                 }
                 lsum[c] += psum;
@@ -536,7 +572,7 @@ paged_prefill_mfma_kernel(PrefillParams p) {
             typedef short v8i16_t __attribute__((ext_vector_type(8)));
 #pragma unroll
             for (int hp = 0; hp < NH / 2; ++hp) {
-                const int voff = DMA ? 32 * hp * KROW + vrow * KROW + (((2 * j + ((r16 >> 1) & 1)) ^ swz(vrow)) << 4) + (r16 & 1) * 8
+                const int voff = DMA ? 32 * hp * KROW + vrow * KROW + (((2 * j + ((r16 >> 1) & 1)) ^ swz_v(vrow)) << 4) + (r16 & 1) * 8
                                      : 32 * hp * KROW + rd_v + j * 32;
                 const v4i16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(vb + voff));
                 const v4i16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(vb + (voff + 16 * KROW)));
@@ -616,7 +652,9 @@ bool prefill_mfma_supported(const DecodeArgs& a, int max_q_len) {
     return a.cu_q_lens != nullptr && max_q_len > 0 && (a.d == 128 || a.d == 64) && a.bs == BS &&
            is_16bit_float(a.q_dtype) &&
            (a.kv_dtype == a.q_dtype || a.kv_dtype == AICOMP_KV_FP8_E4M3) && group >= 1 &&
-           a.scale > 0.f && a.num_seqs <= 65535 && ((uintptr_t)a.query % 16 == 0) &&
+           // the score multiplier is rounded into Q: fp16 queries keep it within a range where
+           // q * multiplier stays a normal fp16 number for ordinary q (bf16 has float's range)
+           a.scale > 0.f && (a.q_dtype == AICOMP_KV_BF16 || (a.scale >= 0x1p-12f && a.scale <= 0x1p8f)) && a.num_seqs <= 65535 && ((uintptr_t)a.query % 16 == 0) &&
            ((uintptr_t)a.out % 16 == 0) && ((uintptr_t)a.k_pool % 16 == 0) &&
            ((uintptr_t)a.v_pool % 16 == 0);
 }
