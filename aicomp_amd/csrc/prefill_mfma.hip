@@ -474,6 +474,17 @@ paged_prefill_mfma_kernel(PrefillParams p) {
                 for (int c = 0; c < R; ++c)
                     sa[h][c] = E::mfma(a[h], qf[c][s], sa[h][c]);
         }
+        // Issue order of the block above: the K operand reads run two k-slots ahead of the MFMAs
+        // that consume them, so a wave that has the SIMD to itself for a while (its neighbour
+        // waiting at the barrier or in its softmax) does not stall on every operand.
+        if constexpr (DMA && DH == 128) {        // (head_dim 64 runs three workgroups per CU: no registers to spare)
+            __builtin_amdgcn_sched_group_barrier(0x100, NSL > 1 ? 2 * NH : NH, 0);       // DS reads
+#pragma unroll
+            for (int s = 0; s < NSL; ++s) {
+                __builtin_amdgcn_sched_group_barrier(0x008, NH * R, 0);                  // MFMA
+                if (s + 2 < NSL) __builtin_amdgcn_sched_group_barrier(0x100, NH, 0);
+            }
+        }
         // Online softmax: the scores arrive as s - m in the exponent's units (multiplier in Q, -m in
         // the accumulators' starting value), so a probability is one exponential.  The max is moved
         // lazily: the exponentials are first taken against the current max, and as long as a lane's
@@ -581,6 +592,15 @@ paged_prefill_mfma_kernel(PrefillParams p) {
 #pragma unroll
                 for (int c = 0; c < R; ++c)
                     O[c][j] = E::mfma(a, pf[c][hp], O[c][j]);
+            }
+        }
+        // same for the V operand reads: two output tiles ahead of their MFMAs
+        if constexpr (DMA && DH == 128) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * NH, 1);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                __builtin_amdgcn_sched_group_barrier(0x008, (NH / 2) * R, 1);
+                if (j + 2 < NJ) __builtin_amdgcn_sched_group_barrier(0x100, NH, 1);
             }
         }
     };
