@@ -176,9 +176,8 @@ static int resolve_parts(int64_t rows, int hkv, int bs, int max_blocks, int& par
 }
 
 static bool streamk_shape(int batch, int hq, int hkv, int d, int bs, int q_dtype, int kv_dtype) {
-    return d == 128 && bs == 16 && is_16bit_float(q_dtype) &&
-           (kv_dtype == q_dtype || kv_dtype == AICOMP_KV_FP8_E4M3) && hq / hkv <= 16 &&
-           batch <= 1024;
+    return ((d == 128 && hq / hkv <= 16) || (d == 64 && hq / hkv <= 8)) && bs == 16 && is_16bit_float(q_dtype) &&
+           (kv_dtype == q_dtype || kv_dtype == AICOMP_KV_FP8_E4M3) && batch <= 1024;
 }
 
 size_t aicomp_paged_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads,

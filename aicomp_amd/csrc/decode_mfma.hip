@@ -282,8 +282,8 @@ __device__ __forceinline__ uint2 quant8_fp8(const uint4& x, float scale) {
 // (context_lens - 1) takes its K/V row from new_key / new_value instead of what was loaded from
 // the pool, and writes it to the pool (the append itself).  No other wave of the launch reads
 // that token.  A tile row is one token (16 lanes of 8 elements), or with PAIR half a row (8 lanes).
-template <typename E, bool FP8, bool PAIR>
-__device__ __forceinline__ void inject_new_row_grid(TileRegs<FP8>& kr, TileRegs<FP8>& vr, const MfmaParams& p,
+template <typename E, bool FP8, bool PAIR, typename Params>
+__device__ __forceinline__ void inject_new_row_grid(TileRegs<FP8>& kr, TileRegs<FP8>& vr, const Params& p,
                                                     int seq, int kvh, int lane, int tile_start, int len,
                                                     const int64_t (&bb)[4]) {
     constexpr int DQ = PAIR ? 64 : D;
@@ -575,20 +575,28 @@ __device__ __forceinline__ void inject_new_row(TileRegs<FP8>& kr, TileRegs<FP8>&
     }
 }
 
+template <int TT>
 __device__ __forceinline__ int sk_tiles(int len, int max_blocks) {
     len = min(max(len, 0), max_blocks * BS);
-    return (len + TILE - 1) / TILE;
+    return (len + TT - 1) / TT;
 }
 
 
-template <typename E, bool FP8>
+// PAIR: head_dim 64 as rows of token pairs (see paged_decode_mfma_kernel): a tile is 64 tokens in
+// four blocks, every head takes two B-operand columns (one per token parity), and a flush writes
+// one partial per column, of which only the 64 elements of the column's own token are kept.
+template <typename E, bool FP8, bool PAIR>
 __global__ void __launch_bounds__(256, 1)     // one workgroup per CU: a wave may use the whole register file
 streamk_decode_kernel(StreamKParams p) {
+    constexpr int DQ = PAIR ? 64 : D;            // head_dim of the tensors
+    constexpr int TT = PAIR ? 2 * TILE : TILE;   // tokens per tile
+    constexpr int BPT = TT / BS;                 // blocks per tile
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r16 = lane & 15, g4 = lane >> 4;
     const int G = p.group, B = p.num_seqs;
+    const int ncol = PAIR ? 2 * G : G;           // B-operand columns in use
 
     __shared__ __attribute__((aligned(16))) unsigned char lds[NWAVES * KTILE_BYTES];
     __shared__ int prefix[SK_MAX_SEQS + 1];     // prefix[s] = tiles of the sequences before s
@@ -599,7 +607,7 @@ streamk_decode_kernel(StreamKParams p) {
     if (B <= 64) {
         // every wave scans for itself and reads back only what it wrote: no barrier (the
         // four waves write identical values to the same words)
-        const int mine = lane < B ? sk_tiles(p.context_lens[lane], p.max_blocks) : 0;
+        const int mine = lane < B ? sk_tiles<TT>(p.context_lens[lane], p.max_blocks) : 0;
         int inc = mine;
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) {
@@ -614,7 +622,7 @@ streamk_decode_kernel(StreamKParams p) {
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const int sidx = 4 * tid + k;
-            loc[k] = sidx < B ? sk_tiles(p.context_lens[sidx], p.max_blocks) : 0;
+            loc[k] = sidx < B ? sk_tiles<TT>(p.context_lens[sidx], p.max_blocks) : 0;
             sum += loc[k];
         }
         int inc = sum;
@@ -674,14 +682,26 @@ streamk_decode_kernel(StreamKParams p) {
     // raw query rows of (sequence, KV head); columns beyond the group are zeroed by q_operand
     // only when the rows are used, so that issuing the loads never waits for them
     auto load_q = [&](int sq, int kh, uint4 (&q)[4]) {
-        const uint4* qp = (const uint4*)((const uint16_t*)p.query +
-                                         ((int64_t)sq * p.hq + kh * G + min(r16, G - 1)) * D + 8 * g4);
+        if constexpr (PAIR) {
+            // column c = (head c / 2, parity c % 2): k-slot s covers row elements 32s + 8 g4 .., which are
+            // the query's elements (32s + 8 g4) % 64 when the slot lies in the column's own half of the row
+            const uint16_t* qrow = (const uint16_t*)p.query + ((int64_t)sq * p.hq + kh * G + min(r16 >> 1, G - 1)) * DQ;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) q[s] = qp[s * 4];
+            for (int s = 0; s < 4; ++s) q[s] = *(const uint4*)(qrow + ((32 * s + 8 * g4) & 63));
+        } else {
+            const uint4* qp = (const uint4*)((const uint16_t*)p.query +
+                                             ((int64_t)sq * p.hq + kh * G + min(r16, G - 1)) * D + 8 * g4);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) q[s] = qp[s * 4];
+        }
     };
     auto q_operand = [&](const uint4 (&raw)[4], uint4 (&q)[4]) {
 #pragma unroll
-        for (int s = 0; s < 4; ++s) q[s] = r16 < G ? raw[s] : make_uint4(0, 0, 0, 0);
+        for (int s = 0; s < 4; ++s) {
+            bool use = r16 < ncol;
+            if constexpr (PAIR) use = use && ((32 * s + 8 * g4 >= 64) == ((r16 & 1) != 0));
+            q[s] = use ? raw[s] : make_uint4(0, 0, 0, 0);
+        }
     };
     auto load_tab = [&](int sq, int first_block) {
         const int32_t* table = p.block_table + (int64_t)sq * p.block_table_stride;
@@ -692,32 +712,44 @@ streamk_decode_kernel(StreamKParams p) {
     uint4 qf[4];
     uint4 qraw[4];
     load_q(seq, kvh, qraw);
-    int tab = load_tab(seq, 2 * t);
+    int tab = load_tab(seq, BPT * t);
     TileRegs<FP8> kr, vr;
+    // the blocks of a tile out of a table slice held one entry per lane
+    auto slice_blocks = [&](int slice, int first, int64_t (&bb)[4]) {
+#pragma unroll
+        for (int j = 0; j < BPT; ++j) bb[j] = clamp_block(__builtin_amdgcn_readlane(slice, first + j), p.num_blocks);
+    };
+    auto load_kv = [&](const int64_t (&bb)[4], int kh) {
+        if constexpr (PAIR) {
+            load_tile_pair<FP8>(kr, p.k_pool, bb[0], bb[1], bb[2], bb[3], p.hkv, kh, lane);
+            load_tile_pair<FP8>(vr, p.v_pool, bb[0], bb[1], bb[2], bb[3], p.hkv, kh, lane);
+        } else {
+            load_tile<FP8>(kr, p.k_pool, bb[0], bb[1], p.hkv, kh, lane);
+            load_tile<FP8>(vr, p.v_pool, bb[0], bb[1], p.hkv, kh, lane);
+        }
+    };
     {
         __builtin_amdgcn_s_waitcnt(0x0F70);                        // Q and table have landed
         q_operand(qraw, qf);
-        const int64_t b0 = clamp_block(__builtin_amdgcn_readlane(tab, 0), p.num_blocks);
-        const int64_t b1 = clamp_block(__builtin_amdgcn_readlane(tab, 1), p.num_blocks);
-        load_tile<FP8>(kr, p.k_pool, b0, b1, p.hkv, kvh, lane);
-        load_tile<FP8>(vr, p.v_pool, b0, b1, p.hkv, kvh, lane);
+        int64_t bb[4] = {0, 0, 0, 0};
+        slice_blocks(tab, 0, bb);
+        load_kv(bb, kvh);
     }
 
     for (int64_t g = g0; g < g1 && seq < B;) {
         const int len = min(p.context_lens[seq], p.max_blocks * BS);
-        const int blk_base = 2 * t;
+        const int blk_base = BPT * t;
         const int32_t* table = p.block_table + (int64_t)seq * p.block_table_stride;
         int tab_first = 0;
         const float cmul = p.qk_mul * (FP8 ? p.k_scale[kvh] : 1.f);
-        auto tile_blocks = [&](int k, int64_t& b0, int64_t& b1) {      // k-th tile of the segment
-            const int i0 = 2 * k;
+        auto tile_blocks = [&](int k, int64_t (&bb)[4]) {              // k-th tile of the segment
+            const int i0 = BPT * k;
             if (i0 - tab_first >= 64) {
                 tab_first = i0;
                 tab = (blk_base + i0 + lane < p.max_blocks) ? table[blk_base + i0 + lane] : 0;
                 __builtin_amdgcn_s_waitcnt(0x0F70);
             }
-            b0 = clamp_block(__builtin_amdgcn_readlane(tab, i0 - tab_first), p.num_blocks);
-            b1 = clamp_block(__builtin_amdgcn_readlane(tab, i0 + 1 - tab_first), p.num_blocks);
+            slice_blocks(tab, i0 - tab_first, bb);
         };
 
         // the segment after this one (same wave, same KV head): the next sequence with tokens
@@ -740,22 +772,24 @@ streamk_decode_kernel(StreamKParams p) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) st.O[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-        int64_t b0, b1;
+        int64_t bb[4] = {0, 0, 0, 0};
         int k = 0;
         for (; k + 1 < nt; ++k) {
-            tile_blocks(k + 1, b0, b1);
-            process_tile<E, FP8, true, false>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, b0, b1,
-                                           p.hkv, kvh, lane, g4, (t + k) * TILE, len, cmul);
+            tile_blocks(k + 1, bb);
+            process_tile<E, FP8, true, false, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, bb[0], bb[1],
+                                                    p.hkv, kvh, lane, g4, (t + k) * TT, len, cmul, bb[2], bb[3]);
         }
-        const int tile_start = (t + k) * TILE;
+        const int tile_start = (t + k) * TT;
         if (p.new_key != nullptr && t + k == row_tiles - 1) {       // the row's newest token lives here
-            tile_blocks(k, b0, b1);
+            tile_blocks(k, bb);
             // Same rule as the separate one-token append: the row is stored only where the table names a
             // block of the pool and the length fits the table; otherwise the call leaves the pools alone
             // (and attends over what the clamped table entry holds, like the unfused sequence of calls).
-            const int raw_blk = __builtin_amdgcn_readlane(tab, 2 * k + ((len - 1 - tile_start) >> 4) - tab_first);
-            if (p.context_lens[seq] == len && raw_blk >= 0 && raw_blk < p.num_blocks)
-                inject_new_row<E, FP8>(kr, vr, p, seq, kvh, lane, tile_start, len, b0, b1);
+            const int raw_blk = __builtin_amdgcn_readlane(tab, BPT * k + ((len - 1 - tile_start) >> 4) - tab_first);
+            if (p.context_lens[seq] == len && raw_blk >= 0 && raw_blk < p.num_blocks) {
+                if constexpr (PAIR) inject_new_row_grid<E, FP8, true>(kr, vr, p, seq, kvh, lane, tile_start, len, bb);
+                else inject_new_row<E, FP8>(kr, vr, p, seq, kvh, lane, tile_start, len, bb[0], bb[1]);
+            }
         }
         // The segment's last tile always runs the masked body (a full tile simply masks nothing):
         // one prefetching call site, so the prefetched registers need no merging afterwards.
@@ -765,28 +799,29 @@ streamk_decode_kernel(StreamKParams p) {
             __builtin_amdgcn_s_waitcnt(0x0F70);      // next Q rows and table slice (and this tile) have landed
             q_operand(qraw, qn);
             tab_ready = tabn;
-            b0 = clamp_block(__builtin_amdgcn_readlane(tab_ready, 0), p.num_blocks);
-            b1 = clamp_block(__builtin_amdgcn_readlane(tab_ready, 1), p.num_blocks);
-            process_tile<E, FP8, true, true>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, b0, b1,
-                                          p.hkv, nkvh, lane, g4, tile_start, len, cmul);
+            slice_blocks(tab_ready, 0, bb);
+            process_tile<E, FP8, true, true, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, bb[0], bb[1],
+                                                   p.hkv, nkvh, lane, g4, tile_start, len, cmul, bb[2], bb[3]);
         } else {
-            process_tile<E, FP8, false, true>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
-                                           p.hkv, kvh, lane, g4, tile_start, len, cmul);
+            process_tile<E, FP8, false, true, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
+                                                    p.hkv, kvh, lane, g4, tile_start, len, cmul);
         }
 
         // ---- flush: lane (head r16, g4) holds O^T[dim 32*g4 + 8*i + j][head] in O[j][i]
         float lsum = st.lsum;
         lsum += __shfl_xor(lsum, 16);
         lsum += __shfl_xor(lsum, 32);
-        if (r16 < G) {
+        // PAIR: column (head, parity) keeps elements 64 * parity .. + 63 of its accumulator (its own token's
+        // half of the pair rows), i.e. the lanes with g4 / 2 == parity, as a partial of 64 floats
+        if (r16 < ncol && (!PAIR || (g4 >> 1) == (r16 & 1))) {
             const int64_t slot = (int64_t)kvh * (p.waves_per_head + B) + part + seq;
-            float* dst = p.ws_acc + (slot * G + r16) * D + 32 * g4;
+            float* dst = p.ws_acc + (slot * ncol + r16) * DQ + 32 * (PAIR ? (g4 & 1) : g4);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 *(float4*)(dst + 8 * i) = make_float4(st.O[0][i], st.O[1][i], st.O[2][i], st.O[3][i]);
                 *(float4*)(dst + 8 * i + 4) = make_float4(st.O[4][i], st.O[5][i], st.O[6][i], st.O[7][i]);
             }
-            if (g4 == 0) *(float2*)(p.ws_ml + (slot * G + r16) * 2) = make_float2(st.m, lsum);
+            if ((g4 & (PAIR ? 1 : 3)) == 0) *(float2*)(p.ws_ml + (slot * ncol + r16) * 2) = make_float2(st.m, lsum);
         }
         // the waves holding a row's first and last tile tell the merge kernel where its partials are
         if (lane == 0) {
@@ -830,15 +865,48 @@ streamk_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ ws_a
     float* wgt = wgt_all[wv];
     const int64_t row = (int64_t)seq * hkv + kvh;
     uint16_t* o = out + ((int64_t)seq * hq + kvh * group + h) * D;
-    if (context_lens[seq] <= 0) {            // no tiles, no partials: the output row is zero (whole workgroup)
+    // the length and the row's record are requested together (the record of an empty row was never
+    // written and is not used)
+    const int ctx = context_lens[seq];
+    const int first = ws_rows[2 * row], last = ws_rows[2 * row + 1];
+    if (ctx <= 0) {                          // no tiles, no partials: the output row is zero (whole workgroup)
         if (sub == 0) { o[lane] = 0; o[lane + 64] = 0; }
         return;
     }
-    const int first = ws_rows[2 * row], last = ws_rows[2 * row + 1];
     const int np = last - first + 1;
     const int64_t slot0 = (int64_t)kvh * head_slots + first + seq;       // the row's partials: slots slot0 .. slot0 + np - 1
     const float* ml = ws_ml + (slot0 * group + h) * 2;                  // partial i at ml[i * group * 2]
     const float* acc = ws_acc + (slot0 * group + h) * D + lane;         // partial i at acc[i * group * D]
+    if (S == 1 && np <= 8) {
+        // The usual batch: a handful of partials per row.  Their (max, sum) pairs and this lane's
+        // two output dims of each are requested in one go, so the kernel is two memory latencies
+        // deep (record, then partials) instead of four.
+        const int64_t stride = (int64_t)group * D;
+        float2 mlv[8];
+        float a[8], b[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = min(u, np - 1);
+            mlv[u] = *(const float2*)(ml + (int64_t)i * group * 2);
+            a[u] = acc[i * stride];
+            b[u] = acc[i * stride + 64];
+        }
+        float mx = NEG_BIG;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) mx = fmaxf(mx, mlv[u].x);           // repeats of the last partial change nothing
+        float den = 0.f, n0 = 0.f, n1 = 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float f = u < np ? exp2f(mlv[u].x - mx) : 0.f;
+            den = fmaf(f, mlv[u].y, den);
+            n0 = fmaf(f, a[u], n0);
+            n1 = fmaf(f, b[u], n1);
+        }
+        const float inv = den > 0.f ? (v_scale ? v_scale[kvh] : 1.f) / den : 0.f;
+        o[lane] = E::from_f32(n0 * inv);
+        o[lane + 64] = E::from_f32(n1 * inv);
+        return;
+    }
     // every wave of a head computes the row's max, denominator and weights for itself (np / 64 loads per lane)
     float mx = NEG_BIG;
     for (int i = lane; i < np; i += 64) mx = fmaxf(mx, ml[(int64_t)i * group * 2]);
@@ -883,6 +951,49 @@ streamk_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ ws_a
     o[lane + 64] = E::from_f32(n1 * inv);
 }
 
+// Merge for head_dim 64 (pair rows): a row's partials are np waves x two token parities, 64 floats
+// each; one wave per head, lane = output dim.  Entry e = (part e / 2, parity e % 2).
+template <typename E>
+__global__ void __launch_bounds__(512)
+streamk_reduce_pair_kernel(uint16_t* __restrict__ out, const float* __restrict__ ws_acc,
+                           const float* __restrict__ ws_ml, const int* __restrict__ ws_rows,
+                           const int32_t* __restrict__ context_lens, int hq, int hkv, int group,
+                           const float* __restrict__ v_scale, int head_slots) {
+    const int kvh = blockIdx.x, seq = blockIdx.y, h = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int ncol = 2 * group;
+    const int64_t row = (int64_t)seq * hkv + kvh;
+    uint16_t* o = out + ((int64_t)seq * hq + kvh * group + h) * 64;
+    const int ctx = context_lens[seq];
+    const int first = ws_rows[2 * row], last = ws_rows[2 * row + 1];
+    if (ctx <= 0) { o[lane] = 0; return; }
+    const int ne = 2 * (last - first + 1);
+    const int64_t col0 = ((int64_t)kvh * head_slots + first + seq) * ncol + 2 * h;     // entry e: column col0 + (e / 2) * ncol + e % 2
+    auto col = [&](int e) { return col0 + (int64_t)(e >> 1) * ncol + (e & 1); };
+    float mx = NEG_BIG;
+    for (int e = lane; e < ne; e += 64) mx = fmaxf(mx, ws_ml[col(e) * 2]);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+    float den = 0.f, num = 0.f;
+    for (int e0 = 0; e0 < ne; e0 += 8) {                     // eight entries in flight per step
+        float2 ml[8];
+        float a[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int64_t c = col(min(e0 + u, ne - 1));
+            ml[u] = *(const float2*)(ws_ml + c * 2);
+            a[u] = ws_acc[c * 64 + lane];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float f = e0 + u < ne ? exp2f(ml[u].x - mx) : 0.f;
+            den = fmaf(f, ml[u].y, den);
+            num = fmaf(f, a[u], num);
+        }
+    }
+    const float inv = den > 0.f ? (v_scale ? v_scale[kvh] : 1.f) / den : 0.f;
+    o[lane] = E::from_f32(num * inv);
+}
+
 }  // namespace
 
 // head_dim 128, or head_dim 64 handled as rows of token pairs (two B-operand columns per head,
@@ -900,12 +1011,14 @@ bool decode_mfma_supported(const DecodeArgs& a) {
 
 bool decode_streamk_supported(const DecodeArgs& a) {
     // every KV head needs at least one wave of the 4 x CUs the schedule launches
-    return decode_mfma_supported(a) && a.d == D && a.rows <= SK_MAX_SEQS && a.hkv <= 256;
+    return decode_mfma_supported(a) && a.rows <= SK_MAX_SEQS && a.hkv <= 256;
 }
 
+// per slot one partial per B-operand column: G columns of D + 2 floats, or 2 G columns of 64 + 2 (head_dim 64)
 size_t decode_streamk_workspace_bytes(int64_t rows, int hq, int hkv, int d) {
     const int64_t slots = SK_MAX_WAVES + rows * hkv;
-    return (size_t)slots * (hq / hkv) * (size_t)(d + 2) * sizeof(float) + (size_t)rows * hkv * 2 * sizeof(int);
+    const int ncol = d == 64 ? 2 * (hq / hkv) : hq / hkv;
+    return (size_t)slots * ncol * (size_t)(d + 2) * sizeof(float) + (size_t)rows * hkv * 2 * sizeof(int);
 }
 
 int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
@@ -938,17 +1051,35 @@ int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
     p.k_scale = a.k_scale; p.v_scale = a.v_scale;
     p.num_waves = wgs * NWAVES;
     p.waves_per_head = p.num_waves / a.hkv;
+    const bool pair = a.d == 64;
+    const int ncol = pair ? 2 * group : group;
     p.ws_acc = (float*)workspace;
-    p.ws_ml = p.ws_acc + slots * group * D;
-    p.ws_rows = (int*)(p.ws_ml + slots * group * 2);
+    p.ws_ml = p.ws_acc + slots * ncol * a.d;
+    p.ws_rows = (int*)(p.ws_ml + slots * ncol * 2);
     p.new_key = (const uint16_t*)a.new_key; p.new_value = (const uint16_t*)a.new_value;
     p.new_token_stride = a.new_token_stride; p.new_head_stride = a.new_head_stride;
     const bool fp8 = a.kv_dtype == AICOMP_KV_FP8_E4M3, f16 = a.q_dtype == AICOMP_KV_F16;
-    if (f16 && fp8) hipLaunchKernelGGL((streamk_decode_kernel<F16Fmt, true>), dim3(wgs), dim3(256), 0, a.stream, p);
-    else if (f16) hipLaunchKernelGGL((streamk_decode_kernel<F16Fmt, false>), dim3(wgs), dim3(256), 0, a.stream, p);
-    else if (fp8) hipLaunchKernelGGL((streamk_decode_kernel<Bf16Fmt, true>), dim3(wgs), dim3(256), 0, a.stream, p);
-    else hipLaunchKernelGGL((streamk_decode_kernel<Bf16Fmt, false>), dim3(wgs), dim3(256), 0, a.stream, p);
+#define AICOMP_LAUNCH_SK(E, PAIR)                                                                                  \
+    do {                                                                                                           \
+        if (fp8) hipLaunchKernelGGL((streamk_decode_kernel<E, true, PAIR>), dim3(wgs), dim3(256), 0, a.stream, p);  \
+        else hipLaunchKernelGGL((streamk_decode_kernel<E, false, PAIR>), dim3(wgs), dim3(256), 0, a.stream, p);    \
+    } while (0)
+    if (pair) { if (f16) AICOMP_LAUNCH_SK(F16Fmt, true); else AICOMP_LAUNCH_SK(Bf16Fmt, true); }
+    else { if (f16) AICOMP_LAUNCH_SK(F16Fmt, false); else AICOMP_LAUNCH_SK(Bf16Fmt, false); }
+#undef AICOMP_LAUNCH_SK
     AICOMP_HIP_LAUNCH_CHECK();
+    if (pair) {
+        if (f16)
+            hipLaunchKernelGGL(streamk_reduce_pair_kernel<F16Fmt>, dim3(a.hkv, (unsigned)a.rows), dim3(64 * group), 0,
+                               a.stream, (uint16_t*)a.out, p.ws_acc, p.ws_ml, p.ws_rows, a.context_lens, a.hq, a.hkv,
+                               group, a.v_scale, p.waves_per_head + (int)a.rows);
+        else
+            hipLaunchKernelGGL(streamk_reduce_pair_kernel<Bf16Fmt>, dim3(a.hkv, (unsigned)a.rows), dim3(64 * group), 0,
+                               a.stream, (uint16_t*)a.out, p.ws_acc, p.ws_ml, p.ws_rows, a.context_lens, a.hq, a.hkv,
+                               group, a.v_scale, p.waves_per_head + (int)a.rows);
+        AICOMP_HIP_LAUNCH_CHECK();
+        return AICOMP_KV_OK;
+    }
     // waves per head in the merge: one, unless rows are few and long (many partials per row)
     const int64_t per_row = (int64_t)p.waves_per_head / a.rows + 2;
     const int sub = per_row > 8 ? 16 / group : 1;

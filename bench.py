@@ -195,7 +195,7 @@ def run_decode_config(name, steps, warmup, dev):
         "kv_dtype": str(w.k_pool.dtype).replace("torch.", ""),
     }
     mfma_shape = (w.shape.head_dim in (64, 128) and w.shape.block_size == 16 and qd.dtype in (torch.bfloat16, torch.float16))
-    balanced = mfma_shape and w.shape.head_dim == 128 and (S - npre) <= 1024
+    balanced = mfma_shape and (S - npre) <= 1024
     res["roofline"] = {
         "kernel": ("streamk_decode_kernel + streamk_reduce_kernel" if balanced else
                    "paged_decode_mfma_kernel + split_reduce_kernel" if mfma_shape else
@@ -408,7 +408,7 @@ def profile_target(which, steps, warmup, dev):
         return
     name = {"decode": "llama3_8b_decode", "append": "chunked_prefill_mixed", "prefill": "chunked_prefill_mixed",
             "decode_fp8": "llama3_70b_decode_fp8", "decode_long": "long_context_skewed",
-            "rope": "chunked_prefill_mixed"}[which]
+            "decode_d64": "llama32_1b_decode", "rope": "chunked_prefill_mixed"}[which]
     w = workloads.make_workload(name, device=dev)
     ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping, w.k_scale, w.v_scale)
     npre = w.num_prefill_seqs
@@ -496,7 +496,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
-    ap.add_argument("--only", choices=["decode", "append", "copy", "prefill", "decode_fp8", "decode_long", "rope", "sample"],
+    ap.add_argument("--only", choices=["decode", "append", "copy", "prefill", "decode_fp8", "decode_long", "decode_d64", "rope", "sample"],
                     help="profiling target: launch just this kernel --steps times (no JSON line)")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -15,18 +15,19 @@ TILE, BS = 32, 16
 SK_MAX_WAVES = 4096
 
 
-def tiles_of(length, max_blocks):
+def tiles_of(length, max_blocks, tile=TILE):
+    """Tiles of a row: 32 tokens at head_dim 128, 64 tokens (32 pair rows) at head_dim 64."""
     length = min(max(length, 0), max_blocks * BS)
-    return (length + TILE - 1) // TILE
+    return (length + tile - 1) // tile
 
 
-def schedule(context_lens, hkv, num_waves, max_blocks):
+def schedule(context_lens, hkv, num_waves, max_blocks, tile=TILE):
     """-> (segments, head_slots): segments are (kvh, part, seq, first_tile, n_tiles, slot)."""
     B = len(context_lens)
     wph = num_waves // hkv
     prefix = [0]
     for c in context_lens:
-        prefix.append(prefix[-1] + tiles_of(c, max_blocks))
+        prefix.append(prefix[-1] + tiles_of(c, max_blocks, tile))
     N = prefix[B]
     W = min(wph, N)
     head_slots = wph + B
@@ -60,9 +61,9 @@ def schedule(context_lens, hkv, num_waves, max_blocks):
     return segs, head_slots
 
 
-def check(context_lens, hkv, num_waves, max_blocks):
+def check(context_lens, hkv, num_waves, max_blocks, tile=TILE):
     B = len(context_lens)
-    segs, head_slots = schedule(context_lens, hkv, num_waves, max_blocks)
+    segs, head_slots = schedule(context_lens, hkv, num_waves, max_blocks, tile)
     # the scratch the library asks for: SK_MAX_WAVES + rows * hkv slots
     limit = SK_MAX_WAVES + B * hkv
     slots = [s[5] for s in segs]
@@ -72,7 +73,7 @@ def check(context_lens, hkv, num_waves, max_blocks):
     for kvh, part, seq, t, nt, slot in segs:
         rows.setdefault((seq, kvh), []).append((t, nt, part, slot))
     for seq in range(B):
-        want = tiles_of(context_lens[seq], max_blocks)
+        want = tiles_of(context_lens[seq], max_blocks, tile)
         for kvh in range(hkv):
             got = sorted(rows.get((seq, kvh), []))
             if want == 0:
@@ -104,7 +105,7 @@ def test_random_batches(seed):
             lens = [rnd.randint(0, max_blocks * BS + 40) for _ in range(B)]     # some beyond the table
         else:
             lens = [rnd.randint(1, max_blocks * BS) for _ in range(B)]
-        check(lens, hkv, 1024, max_blocks)
+        check(lens, hkv, 1024, max_blocks, rnd.choice([32, 64]))
 
 
 def test_corner_cases():
@@ -117,3 +118,4 @@ def test_corner_cases():
     check([100] * 1024, 256, 1024, 8)                   # four waves per head, 1024 rows
     check([100] * 1024, 3, 1024, 8)                     # waves left over (1024 = 3 * 341 + 1)
     check([17] * 10, 8, 4096, 2)                        # the largest launch the scratch is sized for
+    check([0, 63, 64, 65, 4096], 8, 1024, 256, tile=64)  # head_dim 64: tiles of 64 tokens

@@ -458,8 +458,8 @@ def test_fused_append_in_the_grid_kernel_edge_positions(device, d, kv, ps):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("hkv,group", [(8, 4), (3, 2), (16, 1)])
-def test_balanced_schedule_records_the_parts_the_host_model_predicts(hkv, group):
+@pytest.mark.parametrize("hkv,group,D", [(8, 4, 128), (3, 2, 128), (16, 1, 128), (8, 4, 64), (2, 8, 64)])
+def test_balanced_schedule_records_the_parts_the_host_model_predicts(hkv, group, D):
     """The main kernel of the balanced schedule tells the merge kernel, per (sequence, KV head)
     row, which of the head's parts hold the row's first and last tile.  tests/test_decode_schedule.py
     models the schedule on the host and checks its invariants (coverage, distinct slots, bounds);
@@ -469,7 +469,8 @@ def test_balanced_schedule_records_the_parts_the_host_model_predicts(hkv, group)
     from test_decode_schedule import SK_MAX_WAVES, schedule, tiles_of
     dev = torch.device("cuda:0")
     g = torch.Generator().manual_seed(11 + hkv)
-    B, D, hq = 37, 128, hkv * group
+    B, hq = 37, hkv * group
+    tile, ncol = (64, 2 * group) if D == 64 else (32, group)       # head_dim 64: pair rows, two columns per head
     lens = torch.randint(1, 3000, (B,), generator=g).tolist()
     lens[3] = 0; lens[4] = 0; lens[20] = 1; lens[36] = 33
     need = [max(1, math.ceil(c / 16)) for c in lens]
@@ -490,18 +491,21 @@ def test_balanced_schedule_records_the_parts_the_host_model_predicts(hkv, group)
     ops.paged_decode_attn(out, q, k, v, table.to(dev), cl, 1 / math.sqrt(D), None, None, workspace=ws)
     torch.cuda.synchronize()
     slots = SK_MAX_WAVES + B * hkv
-    off = slots * group * D + slots * group * 2                 # partial outputs, then (max, sum) pairs
+    off = slots * ncol * D + slots * ncol * 2                   # partial outputs, then (max, sum) pairs
     assert nbytes >= (off + B * hkv * 2) * 4
     rec = ws.view(torch.int32)[off:off + B * hkv * 2].reshape(B, hkv, 2).cpu()
     num_waves = 4 * torch.cuda.get_device_properties(0).multi_processor_count
-    segs, _ = schedule(lens, hkv, num_waves, max_blocks)
+    segs, _ = schedule(lens, hkv, num_waves, max_blocks, tile)
     first, last = {}, {}
     for kvh, part, seq, t, nt, slot in segs:
         if t == 0:
             first[(seq, kvh)] = part
-        if t + nt == tiles_of(lens[seq], max_blocks):
+        if t + nt == tiles_of(lens[seq], max_blocks, tile):
             last[(seq, kvh)] = part
     for s in range(B):
         for h in range(hkv):
             if lens[s] > 0:
                 assert (int(rec[s, h, 0]), int(rec[s, h, 1])) == (first[(s, h)], last[(s, h)]), (s, h)
+    # and the result itself, against the oracle
+    want = orc.paged_decode_attn(raw(q), raw(k), raw(v), table.numpy(), lens, 1 / math.sqrt(D), "bf16", "bf16")
+    assert_close_attn(to_f64(out), want, BF16_ATOL, BF16_RTOL, f"balanced schedule D {D}")
