@@ -56,3 +56,16 @@ def test_ops_refuse_cpu_tensors():
     x = torch.zeros(1, 1, 64, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError):
         ops.kv_append(x, x, k, k, torch.zeros(1, dtype=torch.int64))
+
+
+def test_prefill_kernel_waits_for_its_tile_loads_before_the_step_barrier():
+    """The direct-to-LDS tile of a step is loaded by all four waves, and the compiler's own waits only
+    order a wave's loads against that same wave's later reads; the kernel therefore has to wait for its
+    outstanding loads itself right before the barrier that opens the step.  Losing that line gives a wrong
+    result once in some hundred runs, which no parity test catches reliably, so the source is checked."""
+    src = open(os.path.join(ROOT, "aicomp_amd", "csrc", "prefill_mfma.hip")).read()
+    code = re.sub(r"//[^\n]*", "", src)
+    step = code[code.index("auto step = "):]
+    first_barrier = step.index("__syncthreads()")
+    before = re.sub(r"\s+", " ", step[:first_barrier]).strip()
+    assert before.endswith("if constexpr (DMA) { __builtin_amdgcn_s_waitcnt(0x0F70);"), before[-200:]

@@ -251,3 +251,28 @@ def test_prefill_context_shorter_than_chunk_gives_zero_rows(device, dtype):
     keep = np.r_[0:lo, hi:got.shape[0]]
     tol = (BF16_ATOL, BF16_RTOL) if dtype == torch.bfloat16 else (1e-5, 0.0)
     assert_close_attn(to_f64(got)[keep], want[keep], tol[0], tol[1], "chunks beside the inconsistent one")
+
+
+def test_long_prompt_sampled_rows_and_scaling_in_v(device):
+    """One fresh prompt of 4096 tokens at the Llama-3-8B head shape (the size class of the long-prompt
+    bench shapes).  The float64 oracle is run on sampled rows only (a full pass takes minutes on the
+    CPU); on all rows the size-independent property is checked that doubling V doubles the output bit
+    for bit (the probabilities do not depend on V, and a factor of two is exact in bf16)."""
+    n = 4096
+    c = build_case(device, priors=[0], news=[n], hq=32, hkv=8, d=128, seed=31, poison=True)
+    got = run(c)
+    assert torch.isfinite(got.float()).all()
+    c2 = dict(c, v_pool=(c["v_pool"].float() * 2).to(torch.bfloat16))
+    got2 = run(c2)
+    assert torch.equal((got.float() * 2).to(torch.bfloat16).view(torch.int16), got2.view(torch.int16))
+    rng = np.random.default_rng(5)
+    kp = torch.nan_to_num(c["k_pool"].float().cpu(), nan=0.0, posinf=0.0).to(torch.bfloat16)
+    vp = torch.nan_to_num(c["v_pool"].float().cpu(), nan=0.0, posinf=0.0).to(torch.bfloat16)
+    tab = c["table"].cpu().numpy()
+    k = orc.decode_elements(orc.gather_context(raw(kp), tab[0], n), "bf16")
+    v = orc.decode_elements(orc.gather_context(raw(vp), tab[0], n), "bf16")
+    qraw, g64 = raw(c["q"]), to_f64(got)
+    for i in sorted(set([0, 1, 63, 64, 127, 128, 2047, 2048, n - 65, n - 64, n - 1] + rng.integers(0, n, 8).tolist())):
+        qv = orc.decode_elements(qraw[i], "bf16")[None]
+        want = orc.attend_contiguous(qv, k[: i + 1], v[: i + 1], c["scale"])[0]
+        assert_close_attn(g64[i], want, BF16_ATOL, BF16_RTOL, f"row {i}")
