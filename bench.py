@@ -173,7 +173,26 @@ def run_decode_config(name, steps, warmup, dev):
         except Exception as e:                              # a bench figure, not a requirement
             print(f"graph replay not measured for {name}: {e}", file=sys.stderr)
     t_app = a0.elapsed_time(a1) / 20 * 1e-3
-    t_pre = statistics.mean(e[1].elapsed_time(e[2]) for e in evs) * 1e-3 if npre else 0.0
+    t_pre_in_step = statistics.mean(e[1].elapsed_time(e[2]) for e in evs) * 1e-3 if npre else 0.0
+    t_pre = 0.0
+    if npre:
+        # The prefill kernel's average launch duration: launches queued back to back between two
+        # events, after ~30 ms of untimed ones (the first launches after an idle gap run 10-15 %
+        # slower while the clock ramps up, and a pair of events around a single launch inside the
+        # mixed step adds their own stream time; that figure is kept as prefill_in_step_us).
+        pre = lambda: ops.paged_prefill_attn(outp, qp, w.k_pool, w.v_pool, btp, clp, cup, w.scale, max_q_len=max_q)
+        tw = time.perf_counter()
+        while time.perf_counter() - tw < 0.03:
+            for _ in range(8):
+                pre()
+            torch.cuda.synchronize()
+        p0, p1 = _events(2)
+        p0.record()
+        for _ in range(50):
+            pre()
+        p1.record()
+        torch.cuda.synchronize()
+        t_pre = p0.elapsed_time(p1) / 50 * 1e-3
     # a pure decode step is one call (main + merge kernel): its average duration is the region's
     t_dec = statistics.mean(e[2].elapsed_time(e[3]) for e in evs) * 1e-3 if npre else region
     res = {
@@ -203,7 +222,7 @@ def run_decode_config(name, steps, warmup, dev):
         "bound": "hbm", "achieved": res["decode_GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": res["decode_frac_hbm_peak"], "algorithmic_bytes": res["decode_bytes"], "avg_launch_us": res["decode_us"]}
     if npre:
-        res.update({"prefill_us": t_pre * 1e6, "prefill_flops": w.prefill_flops(),
+        res.update({"prefill_us": t_pre * 1e6, "prefill_in_step_us": t_pre_in_step * 1e6, "prefill_flops": w.prefill_flops(),
                     "prefill_TFLOPs": w.prefill_flops() / t_pre / 1e12,
                     "prefill_frac_mfma_peak": w.prefill_flops() / t_pre / 1e12 / MFMA_BF16_PEAK_TFLOPS})
         res["prefill_roofline"] = {
