@@ -3,6 +3,7 @@
 // include/aicomp_kv.h.
 #include "common.h"
 
+#include <stdlib.h>
 #include <string.h>
 
 #include <atomic>
@@ -49,13 +50,38 @@ static int check_common(int hq, int hkv, int d, int bs, int max_blocks, int64_t 
     return AICOMP_KV_OK;
 }
 
-static int auto_partition(int64_t rows, int hkv, int bs, int max_blocks) {
+// shapes the balanced schedule and the matrix-core grid schedule both take
+static bool streamk_shape(int batch, int hq, int hkv, int d, int bs, int q_dtype, int kv_dtype) {
+    return ((d == 128 && hq / hkv <= 16) || (d == 64 && hq / hkv <= 8)) && bs == 16 && is_16bit_float(q_dtype) &&
+           (kv_dtype == q_dtype || kv_dtype == AICOMP_KV_FP8_E4M3) && batch <= 1024;
+}
+
+// A decode call over few, short rows is a chain of launch and memory latencies, not a stream: the
+// balanced schedule (set up for 256 CUs of work, always followed by its merge kernel) then loses to
+// one workgroup per (row, KV head, partition) on the grid schedule, without any merge kernel when
+// no row can be longer than 640 tokens (measured on 1 to 16 rows of 512 and 2048 tokens: 5.4-8.5
+// against 9-13 us, 8-15 against 11-17 us).  "Small" is rows x (table width x block size) at or
+// below AICOMP_KV_SMALL_DECODE_TOKENS (default 32768; 0 keeps every automatic call of a supported
+// shape on the balanced schedule).
+static bool small_call(int64_t rows, int bs, int max_blocks) {
+    long long limit = 32768;
+    if (const char* e = getenv("AICOMP_KV_SMALL_DECODE_TOKENS")) limit = atoll(e);
+    return rows * (int64_t)max_blocks * bs <= limit;
+}
+
+static int auto_partition(int64_t rows, int hkv, int bs, int max_blocks, bool matrix_shape) {
     // Longer partitions amortise a workgroup's start-up and merge; shorter ones give the
     // 256 CUs enough workgroups when there are few (sequence, KV head) rows.
     const int64_t max_ctx = (int64_t)max_blocks * bs;
-    int ps = 256;
-    for (int cand : {1024, 512}) {
-        if (rows * hkv * ((max_ctx + cand - 1) / cand) >= 1024) { ps = cand; break; }
+    int ps;
+    if (matrix_shape && small_call(rows, bs, max_blocks)) {
+        // matrix-core grid schedule: whole rows (a whole number of its 64-token tiles), or 256 tokens
+        ps = max_ctx <= 640 ? (int)((max_ctx + 63) / 64 * 64) : 256;
+    } else {
+        ps = 64;       // vector-ALU kernel on few short rows: spread the call wide
+        for (int cand : {1024, 512, 256, 128}) {
+            if (rows * hkv * ((max_ctx + cand - 1) / cand) >= 1024) { ps = cand; break; }
+        }
     }
     ps = (ps + bs - 1) / bs * bs;
     return ps;
@@ -163,21 +189,16 @@ int aicomp_sample_tokens(int64_t* out, const void* logits, int64_t row_stride, f
 int aicomp_paged_decode_partition_size(int batch, int num_q_heads, int num_kv_heads, int head_dim,
                                        int block_size, int max_blocks_per_seq, int q_dtype,
                                        int kv_dtype) {
-    (void)num_q_heads; (void)head_dim; (void)q_dtype; (void)kv_dtype;
-    if (batch <= 0 || num_kv_heads <= 0 || block_size <= 0 || max_blocks_per_seq <= 0) return 0;
-    return auto_partition(batch, num_kv_heads, block_size, max_blocks_per_seq);
+    if (batch <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || block_size <= 0 || max_blocks_per_seq <= 0) return 0;
+    return auto_partition(batch, num_kv_heads, block_size, max_blocks_per_seq,
+                          streamk_shape(batch, num_q_heads, num_kv_heads, head_dim, block_size, q_dtype, kv_dtype));
 }
 
-static int resolve_parts(int64_t rows, int hkv, int bs, int max_blocks, int& partition_size) {
-    if (partition_size <= 0) partition_size = auto_partition(rows, hkv, bs, max_blocks);
+static int resolve_parts(int64_t rows, int hkv, int bs, int max_blocks, bool matrix_shape, int& partition_size) {
+    if (partition_size <= 0) partition_size = auto_partition(rows, hkv, bs, max_blocks, matrix_shape);
     const int64_t max_ctx = (int64_t)max_blocks * bs;
     int64_t parts = (max_ctx + partition_size - 1) / partition_size;
     return (int)(parts < 1 ? 1 : parts);
-}
-
-static bool streamk_shape(int batch, int hq, int hkv, int d, int bs, int q_dtype, int kv_dtype) {
-    return ((d == 128 && hq / hkv <= 16) || (d == 64 && hq / hkv <= 8)) && bs == 16 && is_16bit_float(q_dtype) &&
-           (kv_dtype == q_dtype || kv_dtype == AICOMP_KV_FP8_E4M3) && batch <= 1024;
 }
 
 size_t aicomp_paged_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads,
@@ -187,9 +208,10 @@ size_t aicomp_paged_decode_workspace_bytes(int batch, int num_q_heads, int num_k
         max_blocks_per_seq <= 0 || num_q_heads % num_kv_heads)
         return 0;
     const bool automatic = partition_size <= 0;
-    const int parts = resolve_parts(batch, num_kv_heads, block_size, max_blocks_per_seq, partition_size);
+    const bool matrix_shape = streamk_shape(batch, num_q_heads, num_kv_heads, head_dim, block_size, q_dtype, kv_dtype);
+    const int parts = resolve_parts(batch, num_kv_heads, block_size, max_blocks_per_seq, matrix_shape, partition_size);
     size_t need = parts <= 1 ? 0 : split_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, parts);
-    if (automatic && streamk_shape(batch, num_q_heads, num_kv_heads, head_dim, block_size, q_dtype, kv_dtype)) {
+    if (automatic && matrix_shape && !small_call(batch, block_size, max_blocks_per_seq)) {
         const size_t sk = decode_streamk_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim);
         if (sk > need) need = sk;
     }
@@ -233,13 +255,14 @@ static int decode_impl(void* out, const void* query, const void* new_key, const 
     a.k_scale = kv_dtype == AICOMP_KV_FP8_E4M3 ? k_scale : nullptr;
     a.v_scale = kv_dtype == AICOMP_KV_FP8_E4M3 ? v_scale : nullptr;
     a.partition_size = partition_size;
-    a.num_parts = resolve_parts(batch, num_kv_heads, block_size, max_blocks_per_seq, a.partition_size);
+    const bool matrix_shape = streamk_shape(batch, num_q_heads, num_kv_heads, head_dim, block_size, q_dtype, kv_dtype);
+    a.num_parts = resolve_parts(batch, num_kv_heads, block_size, max_blocks_per_seq, matrix_shape, a.partition_size);
     a.stream = (hipStream_t)stream;
     // the matrix-core kernels append the new rows themselves when they can read them 16 bytes at a time
     const bool injectable = fused && is_16bit_float(q_dtype) && kv_token_stride % 8 == 0 &&
                             kv_head_stride % 8 == 0 && (uintptr_t)new_key % 16 == 0 &&
                             (uintptr_t)new_value % 16 == 0;
-    if (partition_size == 0 && decode_streamk_supported(a)) {
+    if (partition_size == 0 && decode_streamk_supported(a) && !small_call(batch, block_size, max_blocks_per_seq)) {
         // balanced schedule: equal tile counts per wave, merged by a second kernel
         const size_t need = decode_streamk_workspace_bytes(a.rows, a.hq, a.hkv, a.d);
         AICOMP_REQUIRE(workspace && workspace_bytes >= need, AICOMP_KV_EWORKSPACE,

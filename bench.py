@@ -260,6 +260,50 @@ def planner_bench(dev):
             "note": "StepPlanner.schedule() per decode step, including the enqueue of its one H2D copy"}
 
 
+def small_batch_decode_bench(dev):
+    """Decode calls of the size the reference's own engine issues (Llama-3.2-1B heads, 1 to 8
+    sequences of 512 and 2048 tokens): GPU time per call, measured over replays of a HIP graph that
+    holds 20 calls, so that the host's launch rate stays out of the figure."""
+    import math
+    import torch
+    from aicomp_amd import ops
+    hq, hkv, d = 32, 8, 64
+    out_rows = []
+    for B in (1, 8):
+        for ctx in (512, 2048):
+            nblk = math.ceil(ctx / 16)
+            nb = B * nblk + 1
+            g = torch.Generator().manual_seed(0)
+            table = torch.randperm(nb - 1, generator=g)[: B * nblk].reshape(B, nblk).to(torch.int32).to(dev)
+            k = (torch.randn(nb, hkv, 16, d, device=dev) * 0.5).to(torch.bfloat16)
+            v = (torch.randn(nb, hkv, 16, d, device=dev) * 0.5).to(torch.bfloat16)
+            q = torch.randn(B, hq, d, device=dev).to(torch.bfloat16)
+            o = torch.empty_like(q)
+            cl = torch.full((B,), ctx, dtype=torch.int32, device=dev)
+            call = lambda: ops.paged_decode_attn(o, q, k, v, table, cl, 1 / math.sqrt(d))
+            call()
+            torch.cuda.synchronize()
+            graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+            with torch.cuda.stream(side):
+                call()
+                with torch.cuda.graph(graph, stream=side):
+                    for _ in range(20):
+                        call()
+            torch.cuda.synchronize()
+            for _ in range(3):
+                graph.replay()
+            e0, e1 = _events(2)
+            e0.record()
+            for _ in range(10):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            nbytes = B * (2 * ctx * hkv * d * 2 + 2 * hq * d * 2)
+            out_rows.append({"batch": B, "context": ctx, "us_per_call": round(e0.elapsed_time(e1) / 200 * 1e3, 2),
+                             "kv_bytes": nbytes})
+    return {"shape": "32 query / 8 KV heads, head_dim 64, bf16", "calls": out_rows}
+
+
 def sampler_bench(dev, batch=64, vocab=128256, temperature=0.8, top_k=50, top_p=0.9, reps=20):
     """The step after the attention path: one token per row of [64, 128256] fp32 logits with
     temperature / top-k / top-p (opt_prime/opt_prime/inference.py:786-843).  Beside the kernel, the
@@ -565,6 +609,7 @@ def main():
         "device": device_info(),
         "step_planner": planner_bench(dev),
         "sampler": sampler_bench(dev),
+        "decode_small_batch": small_batch_decode_bench(dev),
         "prefill_other_shapes": prefill_shapes_bench(dev),
     }
     if not args.no_cpu:

@@ -104,7 +104,14 @@ int aicomp_kv_append(const void* key, const void* value,
  *                   from the shape (balanced schedule: every wave gets the same
  *                   number of 32-token tiles); a multiple of block_size otherwise.
  *                   Split work is merged by a second kernel from partial
- *                   (max, sum, output) triples.
+ *                   (max, sum, output) triples.  With 0, a call over few short rows
+ *                   (batch * max_blocks_per_seq * block_size at or below the value of
+ *                   the environment variable AICOMP_KV_SMALL_DECODE_TOKENS, default
+ *                   32768; read at every call) runs one workgroup per (row, KV head,
+ *                   256-token partition) instead, and no merge kernel at all when
+ *                   max_blocks_per_seq * block_size <= 640: such a call is bound by
+ *                   launch and memory latency, not by bandwidth.  The result is the
+ *                   same to within the tolerance between split sizes (2e-3).
  *   workspace       device scratch of at least
  *                   aicomp_paged_decode_workspace_bytes(...) bytes (may be NULL
  *                   when that returns 0), 16-byte aligned.  Its contents need

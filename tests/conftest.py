@@ -18,3 +18,11 @@ def device():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
+
+
+@pytest.fixture(autouse=True)
+def balanced_schedule_for_small_shapes(monkeypatch):
+    """The GPU tests run small shapes with partition_size = 0 to exercise the balanced decode
+    schedule; without this the library would route such calls to the grid schedule (its choice
+    for latency-bound calls).  Tests of that choice delete the variable again."""
+    monkeypatch.setenv("AICOMP_KV_SMALL_DECODE_TOKENS", "0")

@@ -509,3 +509,39 @@ def test_balanced_schedule_records_the_parts_the_host_model_predicts(hkv, group,
     # and the result itself, against the oracle
     want = orc.paged_decode_attn(raw(q), raw(k), raw(v), table.numpy(), lens, 1 / math.sqrt(D), "bf16", "bf16")
     assert_close_attn(to_f64(out), want, BF16_ATOL, BF16_RTOL, f"balanced schedule D {D}")
+
+
+# ------------------------------------------------------------------ latency-bound calls: the library's own choice
+@pytest.mark.parametrize("name,batch,ctx_hi,kv", [("llama3_8b_decode", 1, 500, None), ("llama3_8b_decode", 3, 2000, None),
+                                                 ("llama32_1b_decode", 2, 300, None), ("llama32_1b_decode", 4, 1500, None),
+                                                 ("llama3_70b_decode_fp8", 2, 1100, "fp8")])
+def test_small_calls_take_the_grid_schedule(device, monkeypatch, name, batch, ctx_hi, kv):
+    """With partition_size = 0 a call over few short rows is routed to the grid schedule (whole rows
+    when no row can exceed 640 tokens, 256-token partitions otherwise).  Same numbers as the balanced
+    schedule to the tolerance between split sizes, same pools after the fused append, oracle parity,
+    and the sizing helpers agree with what the call does."""
+    from aicomp_amd import _lib
+    lib = _lib.load()
+    w = workloads.make_workload("x", device=device, seed=11, shape=small(name, batch=batch, ctx_lo=40, ctx_hi=ctx_hi))
+    k0, v0 = w.k_pool.clone(), w.v_pool.clone()
+    balanced = torch.full_like(w.query, float("nan"))           # the autouse fixture forces the balanced schedule
+    ops.paged_decode_attn(balanced, w.query, w.k_pool, w.v_pool, w.block_table, w.context_lens, w.scale,
+                          k_scale=w.k_scale, v_scale=w.v_scale, new_key=w.new_key, new_value=w.new_value)
+    torch.cuda.synchronize()
+    monkeypatch.delenv("AICOMP_KV_SMALL_DECODE_TOKENS")
+    s, mb = w.shape, w.block_table.shape[1]
+    assert batch * mb * 16 <= 32768, "the case is meant to be below the default limit"
+    qd, kd = ops._DT[w.query.dtype], ops._DT[w.k_pool.dtype]
+    ps = lib.aicomp_paged_decode_partition_size(batch, s.num_q_heads, s.num_kv_heads, s.head_dim, 16, mb, qd, kd)
+    assert ps == (-(-mb * 16 // 64) * 64 if mb * 16 <= 640 else 256)
+    parts = -(-mb * 16 // ps)
+    need = lib.aicomp_paged_decode_workspace_bytes(batch, s.num_q_heads, s.num_kv_heads, s.head_dim, 16, mb, qd, kd, 0)
+    assert need == (0 if parts == 1 else batch * s.num_q_heads * parts * (s.head_dim + 2) * 4)
+    out = torch.full_like(w.query, float("nan"))
+    ops.paged_decode_attn(out, w.query, k0, v0, w.block_table, w.context_lens, w.scale,
+                          k_scale=w.k_scale, v_scale=w.v_scale, new_key=w.new_key, new_value=w.new_value)
+    torch.cuda.synchronize()
+    bits = lambda t: t.view(torch.uint8) if t.dtype == torch.float8_e4m3fn else t
+    assert torch.equal(bits(k0), bits(w.k_pool)) and torch.equal(bits(v0), bits(w.v_pool))
+    assert_close_attn(to_f64(out), to_f64(balanced), 2e-3, 0.0, "grid against balanced schedule")
+    assert_close_attn(to_f64(out), oracle_decode(w), BF16_ATOL, BF16_RTOL, "grid schedule against the oracle")
