@@ -92,6 +92,9 @@ class _PagedLayer:
         # row L of this table is the context-length vector of a step that sees L tokens: all
         # sequences share one position, so a decode step takes a view instead of launching a fill
         self.ctx_rows = _ctx_rows(self.blocks_per_seq * block_size + 1, batch, torch.device(device))
+        # the same vector kept on the device and advanced by a kernel, for decode steps that are
+        # replayed from a HIP graph (a replay runs no host code, so it cannot pick another row)
+        self.live_ctx = torch.zeros(batch, dtype=torch.int32, device=device)
         self._decode: Dict[tuple, ops.PreparedDecode] = {}
         self.cu_q_lens = torch.zeros(batch + 1, dtype=torch.int32, device=device)
         self._cu_n = -1
@@ -113,9 +116,11 @@ class _PagedLayer:
         ops.kv_append(rows_k, rows_v, self.k_pool, self.v_pool, slots)
 
     def decode_step(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, pos: int,
-                    group: int, scale: float) -> torch.Tensor:
+                    group: int, scale: float, live: bool = False) -> torch.Tensor:
         """One decode step, append and attention in a single call: query ``[B, Hq, 1, D]``,
-        key/value ``[B, H, 1, D]`` written at position pos."""
+        key/value ``[B, H, 1, D]`` written at position pos.  With ``live`` the position is the
+        device-side counter ``live_ctx`` (advanced here by a one-element-per-sequence kernel), so
+        the step can be captured into a HIP graph and replayed."""
         B, Hq, _, D = query.shape
         if key.shape[1] == self.kv_heads * group and group > 1:
             key, value = key[:, ::group], value[:, ::group]
@@ -126,7 +131,12 @@ class _PagedLayer:
             self._decode[(Hq, query.dtype, scale)] = call
         q = query[:, :, 0, :].contiguous()
         out = torch.empty_like(q)
-        call(out, q, key[:, :, 0, :], value[:, :, 0, :], context_lens=self.ctx_rows[pos + 1])
+        if live:
+            self.live_ctx.add_(1)                 # a fill-type kernel: safe inside a captured graph
+            ctx = self.live_ctx
+        else:
+            ctx = self.ctx_rows[pos + 1]
+        call(out, q, key[:, :, 0, :], value[:, :, 0, :], context_lens=ctx)
         return out.view(B, Hq, 1, D)
 
     def attend(self, query: torch.Tensor, pos: int, scale: float) -> torch.Tensor:
@@ -353,6 +363,7 @@ class CachedScaledDotProductAttention(nn.Module):
         self._store: Optional[_PagedLayer] = None
         self.cache_pos: int = 0
         self._enabled: bool = False
+        self._device_positions: bool = False
         self.kv_manager: Optional[KVCacheManager] = None
 
     # the reference exposes its tensors under these names; here they are the block pools
@@ -379,12 +390,39 @@ class CachedScaledDotProductAttention(nn.Module):
 
     def disable(self) -> None:
         self._enabled = False
+        self._device_positions = False
         self.cache_pos = 0
         self._store = None
+
+    def use_device_positions(self, on: bool = True) -> None:
+        """Keep the decode position on the device (no counterpart in the reference, whose cache
+        position is a Python integer, ``kv_cache.py:372-388``): for callers that capture a decode
+        step into a HIP graph.  A replay runs no Python, so it can neither advance ``cache_pos``
+        nor choose another context-length vector; with this switch a decode step first advances a
+        per-layer device counter and attends with it.  Call it after the prompt has been ingested
+        (it starts the counter at the current ``cache_pos``), capture and replay decode steps,
+        then ``advance(n)`` by the number of replays before the next eager call.  Internal mode
+        only.  A replay past ``max_seq_len`` stores nothing (the kernel's bounds rule) and
+        attends to the full cache."""
+        if on:
+            if self.kv_manager is not None:
+                raise RuntimeError("device positions need the operator's own cache (no kv_manager)")
+            if self._store is None:
+                raise RuntimeError("device positions start from an ingested prompt: run the prefill first")
+            self._store.live_ctx.fill_(self.cache_pos)
+        self._device_positions = on
+
+    def advance(self, steps: int) -> None:
+        """Account on the host for decode steps that were replayed from a graph."""
+        if steps < 0 or self.cache_pos + steps > self.max_seq_len:
+            raise RuntimeError(f"advance({steps}) from position {self.cache_pos} leaves the cache "
+                               f"(max_seq_len {self.max_seq_len})")
+        self.cache_pos += steps
 
     def clear(self) -> None:
         """Reset the write position; the allocation is kept (``kv_cache.py:324-338``)."""
         self.cache_pos = 0
+        self._device_positions = False
 
     def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                 attn_mask: Optional[torch.Tensor] = None, dropout_p: float = 0.0,
@@ -424,8 +462,11 @@ class CachedScaledDotProductAttention(nn.Module):
                 raise RuntimeError(f"cache overflow: position {pos} + {n} new tokens > max_seq_len "
                                    f"{self.max_seq_len}")
             if n == 1 and key.dtype == store.k_pool.dtype:
-                self.cache_pos = pos + 1          # decode step: append fused into the attention call
-                return store.decode_step(query, key, value, pos, self._group, scale)
+                # decode step: append fused into the attention call.  A call that is only being
+                # recorded into a graph executes nothing: the host position stays (see advance()).
+                if not (self._device_positions and torch.cuda.is_current_stream_capturing()):
+                    self.cache_pos = pos + 1
+                return store.decode_step(query, key, value, pos, self._group, scale, live=self._device_positions)
             store.append(key, value, pos, self._group)
         self.cache_pos = pos + n
         # the caller's attn_mask is dropped, as in the reference (kv_cache.py:400-415): decode sees

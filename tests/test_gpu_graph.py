@@ -90,3 +90,78 @@ def test_fused_decode_step_replays_under_a_graph(device, kv_dtype):
         ctx_s += 1
         ctx_e += 1
         _ = (out_s.float() @ out_s.float().transpose(1, 2)).sum().item()
+
+
+@pytest.mark.parametrize("B,d,prompt", [(2, 64, 37), (4, 128, 600)])
+def test_adapter_decode_step_replays_from_a_graph(device, monkeypatch, B, d, prompt):
+    """Two layers of the drop-in operator with device-side positions: one decode step (both layers)
+    is captured once and replayed with new inputs; every replay equals the same step made eagerly by
+    a twin pair of operators, bit for bit, and the host positions agree after ``advance``.  Runs with
+    the library's own schedule choice (these sizes take the grid schedule) and eager work between
+    the replays."""
+    from aicomp_amd import kv_cache as akv
+    monkeypatch.delenv("AICOMP_KV_SMALL_DECODE_TOKENS")
+    hq, g = 8, 4
+    hkv = hq // g
+    gen = torch.Generator().manual_seed(3)
+    mk = lambda n, h: torch.randn(B, h, n, d, generator=gen).to(torch.bfloat16).to(device)
+    expand = lambda t: t.repeat_interleave(g, 1)
+    graph_ops = [akv.CachedScaledDotProductAttention(i, 1024, num_kv_groups=g) for i in range(2)]
+    eager_ops = [akv.CachedScaledDotProductAttention(i, 1024, num_kv_groups=g) for i in range(2)]
+    for op in graph_ops + eager_ops:
+        op.enable()
+    for i in range(2):                                   # prompt, eagerly, same data for the twins
+        q, k, v = mk(prompt, hq), expand(mk(prompt, hkv)), expand(mk(prompt, hkv))
+        a = graph_ops[i](q, k, v, is_causal=True)
+        b = eager_ops[i](q, k, v, is_causal=True)
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    for op in graph_ops:
+        op.use_device_positions()
+    q_s = [torch.zeros(B, hq, 1, d, dtype=torch.bfloat16, device=device) for _ in range(2)]
+    k_s = [torch.zeros(B, hq, 1, d, dtype=torch.bfloat16, device=device) for _ in range(2)]
+    v_s = [torch.zeros(B, hq, 1, d, dtype=torch.bfloat16, device=device) for _ in range(2)]
+    out_s = [None, None]
+
+    def step():
+        for i in range(2):
+            out_s[i] = graph_ops[i](q_s[i], k_s[i], v_s[i])
+
+    # one eager step on the capture stream first (allocates the per-stream scratch), then the capture
+    steps = 5
+    feed = [[(mk(1, hq), expand(mk(1, hkv)), expand(mk(1, hkv))) for _ in range(2)] for _ in range(steps)]
+    want = []
+    for t in range(steps):
+        want.append([eager_ops[i](*feed[t][i]).clone() for i in range(2)])
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        for i in range(2):
+            q_s[i].copy_(feed[0][i][0]); k_s[i].copy_(feed[0][i][1]); v_s[i].copy_(feed[0][i][2])
+        step()                                           # eager: this IS step 0
+        got0 = [o.clone() for o in out_s]
+        side.synchronize()
+        pos_before = [op.cache_pos for op in graph_ops]
+        with torch.cuda.graph(graph, stream=side):
+            step()
+        assert [op.cache_pos for op in graph_ops] == pos_before, "a recorded call is not a step"
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert torch.equal(got0[i].view(torch.int16), want[0][i].view(torch.int16))
+    filler = torch.empty(1 << 24, dtype=torch.uint8, device=device)
+    for t in range(1, steps):
+        for i in range(2):
+            q_s[i].copy_(feed[t][i][0]); k_s[i].copy_(feed[t][i][1]); v_s[i].copy_(feed[t][i][2])
+        filler.fill_(t)                                  # the program's own eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for i in range(2):
+            assert torch.equal(out_s[i].view(torch.int16), want[t][i].view(torch.int16)), f"replay {t}, layer {i}"
+    for op in graph_ops:
+        op.advance(steps - 1)
+    assert [op.cache_pos for op in graph_ops] == [op.cache_pos for op in eager_ops] == [prompt + steps] * 2
+    # the caches hold the same rows, and an eager step after the replays continues from there
+    for i in range(2):
+        assert torch.equal(graph_ops[i].cache_k.view(torch.int16), eager_ops[i].cache_k.view(torch.int16))
+        q, k, v = mk(1, hq), expand(mk(1, hkv)), expand(mk(1, hkv))
+        assert torch.equal(graph_ops[i](q, k, v).view(torch.int16), eager_ops[i](q, k, v).view(torch.int16))
