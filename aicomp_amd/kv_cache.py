@@ -95,6 +95,7 @@ class _PagedLayer:
         # the same vector kept on the device and advanced by a kernel, for decode steps that are
         # replayed from a HIP graph (a replay runs no host code, so it cannot pick another row)
         self.live_ctx = torch.zeros(batch, dtype=torch.int32, device=device)
+        self._ctx_base, self._ctx_pitch = self.ctx_rows.data_ptr(), self.ctx_rows.stride(0) * 4
         self._decode: Dict[tuple, ops.PreparedDecode] = {}
         self.cu_q_lens = torch.zeros(batch + 1, dtype=torch.int32, device=device)
         self._cu_n = -1
@@ -121,23 +122,22 @@ class _PagedLayer:
         key/value ``[B, H, 1, D]`` written at position pos.  With ``live`` the position is the
         device-side counter ``live_ctx`` (advanced here by a one-element-per-sequence kernel), so
         the step can be captured into a HIP graph and replayed."""
-        B, Hq, _, D = query.shape
-        if key.shape[1] == self.kv_heads * group and group > 1:
-            key, value = key[:, ::group], value[:, ::group]
+        Hq = query.shape[1]
         call = self._decode.get((Hq, query.dtype, scale))
         if call is None:
             call = ops.PreparedDecode(self.k_pool, self.v_pool, self.block_table, self.context_lens, Hq,
                                       query.dtype, scale)
             self._decode[(Hq, query.dtype, scale)] = call
-        q = query[:, :, 0, :].contiguous()
-        out = torch.empty_like(q)
         if live:
             self.live_ctx.add_(1)                 # a fill-type kernel: safe inside a captured graph
-            ctx = self.live_ctx
+            ctx = self.live_ctx.data_ptr()
         else:
-            ctx = self.ctx_rows[pos + 1]
-        call(out, q, key[:, :, 0, :], value[:, :, 0, :], context_lens=ctx)
-        return out.view(B, Hq, 1, D)
+            # row pos + 1 of the context-length table, by address (a view tensor costs microseconds)
+            ctx = self._ctx_base + (pos + 1) * self._ctx_pitch
+        if not query.is_contiguous():
+            query = query.contiguous()
+        # [B, Hq, 1, D] has the memory layout of [B, Hq, D]: the call takes the tensors as they are
+        return call.step4d(torch.empty_like(query), query, key, value, group, ctx)
 
     def attend(self, query: torch.Tensor, pos: int, scale: float) -> torch.Tensor:
         """query ``[B, Hq, n, D]`` at positions pos..pos+n (rows already appended)."""

@@ -34,9 +34,20 @@ def _dev(t: torch.Tensor, ref: torch.Tensor, what: str) -> None:
     _req(t.device == ref.device, f"{what} is on {t.device}, expected {ref.device}")
 
 
+# torch's raw-stream getter (what its own compiled-kernel launchers call) costs a fraction of a
+# microsecond; building a torch.cuda.Stream object per call costs about four
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _current_stream(device: torch.device) -> int:
+    if _raw_stream is not None:
+        return _raw_stream(device.index if device.index is not None else torch.cuda.current_device())
+    return torch.cuda.current_stream(device).cuda_stream
+
+
 def _stream(t: torch.Tensor) -> int:
     _req(t.is_cuda, "tensors must live on a ROCm device (there is no CPU path)")
-    return torch.cuda.current_stream(t.device).cuda_stream
+    return _current_stream(t.device)
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -99,7 +110,7 @@ _workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
 def _workspace(device: torch.device, nbytes: int, stream: Optional[int] = None) -> Optional[torch.Tensor]:
     if nbytes == 0:
         return None
-    key = (device.index or 0, torch.cuda.current_stream(device).cuda_stream if stream is None else stream)
+    key = (device.index or 0, _current_stream(device) if stream is None else stream)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
@@ -239,7 +250,7 @@ class PreparedDecode:
              and query.is_contiguous() and out.is_contiguous(),
              f"out/query must be contiguous {self.q_shape} {self.q_dtype} tensors on {self.device}")
         ctx = self.context_lens if context_lens is None else context_lens
-        stream = torch.cuda.current_stream(self.device).cuda_stream
+        stream = _current_stream(self.device)
         ws = _workspace(self.device, self.need, stream)
         ws_ptr, ws_bytes = (None, 0) if ws is None else (ws.data_ptr(), ws.numel())
         if new_key is None:
@@ -256,6 +267,37 @@ class PreparedDecode:
                 out.data_ptr(), query.data_ptr(), new_key.data_ptr(), new_value.data_ptr(),
                 new_key.stride(0), new_key.stride(1), *self._head, ctx.data_ptr(), *self._tail,
                 ws_ptr, ws_bytes, stream)
+        _lib.check(rc, self.lib)
+        return out
+
+    def step4d(self, out: torch.Tensor, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+               group: int, context_lens) -> torch.Tensor:
+        """The fused append + decode call on the operator's own tensors: ``query`` / ``out``
+        ``[B, Hq, 1, D]`` contiguous, ``key`` / ``value`` ``[B, H, 1, D]`` with H = Hkv or
+        Hkv * group (heads repeated ``group`` times, as HF's ``repeat_kv`` leaves them: every
+        group-th head is read).  No view tensors are made: the strides go to the library as they
+        are.  ``context_lens`` is an int32 ``[B]`` tensor on the device, or its device address."""
+        B, Hq, D = self.q_shape
+        hkv = self.kv_shape[1]
+        H = key.shape[1]
+        hstep = group if (group > 1 and H == hkv * group) else 1
+        _req(query.shape == (B, Hq, 1, D) and out.shape == (B, Hq, 1, D) and query.dtype == self.q_dtype
+             and out.dtype == self.q_dtype and query.device == self.device and out.device == self.device
+             and query.is_contiguous() and out.is_contiguous(),
+             f"out/query must be contiguous {(B, Hq, 1, D)} {self.q_dtype} tensors on {self.device}")
+        _req(key.shape == (B, hkv * hstep, 1, D) and value.shape == key.shape and key.dtype == self.q_dtype
+             and value.dtype == self.q_dtype and key.device == self.device and value.device == self.device,
+             f"key/value must both be [{B}, {hkv} or {hkv}*group, 1, {D}] of the query dtype on {self.device}")
+        if key.stride(3) != 1 or key.stride() != value.stride():
+            key, value = key.contiguous(), value.contiguous()
+        stream = _current_stream(self.device)
+        ws = _workspace(self.device, self.need, stream)
+        ws_ptr, ws_bytes = (None, 0) if ws is None else (ws.data_ptr(), ws.numel())
+        rc = self.lib.aicomp_paged_decode_attn_append(
+            out.data_ptr(), query.data_ptr(), key.data_ptr(), value.data_ptr(),
+            key.stride(0), key.stride(1) * hstep, *self._head,
+            context_lens if isinstance(context_lens, int) else context_lens.data_ptr(), *self._tail,
+            ws_ptr, ws_bytes, stream)
         _lib.check(rc, self.lib)
         return out
 
