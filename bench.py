@@ -479,6 +479,24 @@ def profile_target(which, steps, warmup, dev):
         torch.cuda.synchronize()
         print(f"sample: {steps + warmup} launches over [64, 128256] fp32 logits, temperature 0.8, top-k 50, top-p 0.9")
         return
+    if which == "prefill_long":
+        # one fresh prompt of 8192 tokens at the Llama-3-8B head shape (a row of prefill_other_shapes)
+        import math
+        nseq, n, hq, hkv, d = 1, 8192, 32, 8, 128
+        nblk = n // 16
+        g = torch.Generator().manual_seed(0)
+        table = torch.randperm(nblk, generator=g).reshape(1, nblk).to(torch.int32).to(dev)
+        k = (torch.randn(nblk + 1, hkv, 16, d, device=dev) * 0.5).to(torch.bfloat16)
+        v = (torch.randn(nblk + 1, hkv, 16, d, device=dev) * 0.5).to(torch.bfloat16)
+        q = torch.randn(n, hq, d, device=dev).to(torch.bfloat16)
+        o = torch.empty_like(q)
+        cl = torch.full((1,), n, dtype=torch.int32, device=dev)
+        cu = torch.tensor([0, n], dtype=torch.int32, device=dev)
+        for _ in range(warmup + steps):
+            ops.paged_prefill_attn(o, q, k, v, table, cl, cu, 1 / math.sqrt(d), max_q_len=n)
+        torch.cuda.synchronize()
+        print(f"prefill_long: {steps + warmup} launches, {4 * hq * d * (n * (n + 1) // 2)} algorithmic flop per launch")
+        return
     name = {"decode": "llama3_8b_decode", "append": "chunked_prefill_mixed", "prefill": "chunked_prefill_mixed",
             "decode_fp8": "llama3_70b_decode_fp8", "decode_long": "long_context_skewed",
             "decode_d64": "llama32_1b_decode", "rope": "chunked_prefill_mixed"}[which]
@@ -569,7 +587,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
-    ap.add_argument("--only", choices=["decode", "append", "copy", "prefill", "decode_fp8", "decode_long", "decode_d64", "rope", "sample"],
+    ap.add_argument("--only", choices=["decode", "append", "copy", "prefill", "prefill_long", "decode_fp8", "decode_long", "decode_d64", "rope", "sample"],
                     help="profiling target: launch just this kernel --steps times (no JSON line)")
     args = ap.parse_args()
     if args.gpus != 1:
