@@ -26,7 +26,12 @@ def _close(got, want, atol, rtol):
 
 
 @pytest.mark.parametrize("seed", range(4))
-def test_random_decode_and_prefill_shapes(device, seed):
+@pytest.mark.parametrize("schedule", ["balanced", "library"])
+def test_random_decode_and_prefill_shapes(device, monkeypatch, seed, schedule):
+    # "library": the library's own choice of decode schedule for small calls (the suite otherwise
+    # pins automatic calls to the balanced schedule)
+    if schedule == "library":
+        monkeypatch.delenv("AICOMP_KV_SMALL_DECODE_TOKENS")
     rnd = random.Random(100 + seed)
     for trial in range(12):
         nseq = rnd.randint(1, 5)
