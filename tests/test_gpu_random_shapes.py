@@ -66,7 +66,10 @@ def test_random_decode_and_prefill_shapes(device, monkeypatch, seed, schedule):
 
 
 @pytest.mark.parametrize("seed", range(3))
-def test_random_operator_sessions(device, seed):
+@pytest.mark.parametrize("schedule", ["balanced", "library"])
+def test_random_operator_sessions(device, monkeypatch, seed, schedule):
+    if schedule == "library":
+        monkeypatch.delenv("AICOMP_KV_SMALL_DECODE_TOKENS")
     rnd = random.Random(200 + seed)
     torch.manual_seed(200 + seed)
     for trial in range(10):
