@@ -580,6 +580,31 @@ def cpu_baseline(w, budget_s=20.0):
                       f"cpu '{model}', os.cpu_count()={os.cpu_count()}, torch threads={threads}"}
 
 
+def cpu_prefill_baseline(w):
+    """The reference's CPU prefill call (gather -> repeat_kv -> contiguous -> SDPA), restated in
+    oracle/contiguous_ref.py, timed on the host cores for the first chunk of the workload."""
+    import torch
+    from oracle import contiguous_ref as cref
+    n, L = w.new_list[0], w.ctx_list[0]
+    q = w.query[: n].cpu()
+    bt = w.block_table[0].cpu()
+    kp, vp = w.k_pool.cpu(), w.v_pool.cpu()
+    run = lambda: cref.reference_cpu_prefill(q, kp, vp, bt, L, w.scale, compute_dtype=q.dtype)
+    run()
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        run()
+        ts.append(time.perf_counter() - t0)
+    med = sorted(ts)[1]
+    s = w.shape
+    flops = 4 * s.num_q_heads * s.head_dim * (n * (L - n) + n * (n + 1) / 2)
+    return {"value": flops / med / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"first chunk of the workload ({n} new tokens over {L - n} prior ones): gather blocks -> repeat_kv -> "
+                      f"contiguous -> torch SDPA with the chunk's causal mask, {str(q.dtype).replace('torch.', '')}, "
+                      f"1 warm-up, median of 3; {med * 1e3:.1f} ms per pass"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -653,6 +678,8 @@ def main():
                 # the reference's CPU path on the same batch, in the workload's own dtype (fp32 for
                 # the small anchor shape, which is defined on that path); a few seconds each
                 r["cpu_baseline"] = cpu_baseline(ww, budget_s=5.0)
+                if ww.num_prefill_seqs:
+                    r["prefill_cpu_baseline"] = cpu_prefill_baseline(ww)
             del ww
             torch.cuda.empty_cache()
             rnd = lambda v: round(v, 4) if isinstance(v, float) else v

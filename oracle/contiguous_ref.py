@@ -163,3 +163,32 @@ def reference_cpu_decode(query, k_pool, v_pool, block_table, context_lens, scale
         out[b] = F.scaled_dot_product_attention(q, k, v, attn_mask=None, is_causal=False,
                                                 scale=scale)[0, :, 0]
     return out
+
+
+def reference_cpu_prefill(query, k_pool, v_pool, block_table, context_len, scale, compute_dtype=None):
+    """The reference's prefill call for ONE chunk on paged inputs, the way its CPU path runs it:
+    gather the sequence's blocks to a contiguous ``[1, Hkv, L, D]``, ``repeat_kv`` to the query
+    heads (modeling_llama.py:268-277), ``.contiguous()`` (kv_cache.py:391-392) and SDPA
+    (kv_cache.py:404-415).  A chunk that starts the sequence is ``is_causal=True`` as in the
+    reference; a chunk over a prior context gets the causal-within-the-chunk mask this build
+    defines for that case (the reference never issues such a call).  query ``[n, Hq, D]`` (the
+    chunk's tokens, in order), context_len = prior + n; returns ``[n, Hq, D]``."""
+    n, hq, d = query.shape
+    nb, hkv, bs, _ = k_pool.shape
+    g = hq // hkv
+    cd = compute_dtype or query.dtype
+    L = int(context_len)
+    prior = L - n
+    nblk = (L + bs - 1) // bs
+    blocks = block_table[:nblk].long()
+    k = k_pool[blocks].permute(1, 0, 2, 3).reshape(hkv, nblk * bs, d)[:, :L].to(cd)
+    v = v_pool[blocks].permute(1, 0, 2, 3).reshape(hkv, nblk * bs, d)[:, :L].to(cd)
+    k = k[:, None].expand(hkv, g, L, d).reshape(1, hq, L, d).contiguous()
+    v = v[:, None].expand(hkv, g, L, d).reshape(1, hq, L, d).contiguous()
+    q = query.to(cd).permute(1, 0, 2).reshape(1, hq, n, d)
+    if prior == 0:
+        out = F.scaled_dot_product_attention(q, k, v, attn_mask=None, is_causal=True, scale=scale)
+    else:
+        mask = torch.arange(L)[None, :] <= (prior + torch.arange(n))[:, None]
+        out = F.scaled_dot_product_attention(q, k, v, attn_mask=mask, is_causal=False, scale=scale)
+    return out[0].permute(1, 0, 2)

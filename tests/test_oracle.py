@@ -364,3 +364,21 @@ def test_contiguous_store_errors():
     assert st.seq_len == 3
     k3, _ = st.update(1, torch.ones(2, 3, 4), torch.ones(2, 3, 4))   # 3-D input: batch 1 broadcast
     assert k3.shape == (2, 2, 6, 4)
+
+
+@pytest.mark.parametrize("prior,n", [(0, 1), (0, 37), (13, 9), (64, 40)])
+def test_cpu_prefill_restatement_equals_the_paged_oracle(prior, n):
+    """The bench's CPU baseline for chunked prefill (gather -> repeat_kv -> contiguous -> SDPA) gives
+    what the float64 paged oracle gives, for a chunk that starts a sequence (is_causal, as in the
+    reference) and for one over a prior context (this build's causal-within-the-chunk rule)."""
+    torch.manual_seed(prior + n)
+    hq, hkv, d, bs = 6, 2, 16, 16
+    L = prior + n
+    nblk = -(-L // bs)
+    kp, vp = torch.randn(nblk + 3, hkv, bs, d), torch.randn(nblk + 3, hkv, bs, d)
+    tab = torch.randperm(nblk + 3)[:nblk].to(torch.int32)
+    q = torch.randn(n, hq, d)
+    got = cref.reference_cpu_prefill(q, kp, vp, tab, L, 1 / d ** 0.5).double().numpy()
+    want = orc.paged_prefill_attn(q.numpy(), kp.numpy(), vp.numpy(), tab[None].numpy(), [L], np.array([0, n]),
+                                  1 / d ** 0.5, "f32", "f32")
+    assert np.abs(got - want).max() < 2e-6
