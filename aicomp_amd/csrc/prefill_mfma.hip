@@ -150,13 +150,17 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     // chunk, not per item.  Other grids keep the grid order, longest tile of every chunk first.
     int seq = blockIdx.y, qtile = gridDim.z - 1 - blockIdx.z;
     const int nseq = gridDim.y, ntile = gridDim.z, items = nseq * ntile;
+    bool ranked = false;
+    int r_ctx = 0, r_n = 0, r_qb = 0;
     if (p.num_cus > 0 && nseq > 1 && nseq <= 16 && items <= 256) {     // workgroup-uniform
         int* scratch = (int*)(DMA ? dma_k0 : lds);                     // the tile buffers are still unused
         if (tid < nseq) {
-            const int n_t = p.cu_q_lens[tid + 1] - p.cu_q_lens[tid];
+            const int qb_t = p.cu_q_lens[tid];
+            const int n_t = p.cu_q_lens[tid + 1] - qb_t;
             const int ctx_t = min(p.context_lens[tid], p.max_blocks * BS);
             scratch[4 * tid] = ctx_t;
             scratch[4 * tid + 1] = ctx_t - n_t;
+            scratch[4 * tid + 3] = qb_t;
             scratch[4 * tid + 2] = (n_t > 0 && ctx_t >= n_t) ? min(ntile, (n_t + pos_per_wg - 1) / pos_per_wg) : 0;   // tiles with work
         }
         __syncthreads();
@@ -196,12 +200,17 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         __syncthreads();
         seq = __builtin_amdgcn_readfirstlane(scratch[64]);
         qtile = __builtin_amdgcn_readfirstlane(scratch[65]);
+        // the chosen chunk's numbers are in the scratch already: no second trip to memory for them
+        r_ctx = __builtin_amdgcn_readfirstlane(scratch[4 * seq]);
+        r_n = r_ctx - __builtin_amdgcn_readfirstlane(scratch[4 * seq + 1]);
+        r_qb = __builtin_amdgcn_readfirstlane(scratch[4 * seq + 3]);
+        ranked = true;
         __syncthreads();                       // before the first tile is written over the scratch
     }
 
-    const int q_begin = p.cu_q_lens[seq];
-    const int n = p.cu_q_lens[seq + 1] - q_begin;
-    const int ctx = min(p.context_lens[seq], p.max_blocks * BS);
+    const int q_begin = ranked ? r_qb : p.cu_q_lens[seq];
+    const int n = ranked ? r_n : p.cu_q_lens[seq + 1] - q_begin;
+    const int ctx = ranked ? r_ctx : min(p.context_lens[seq], p.max_blocks * BS);
     const int prior = ctx - n;
     const int q0 = qtile * pos_per_wg;
     if (q0 >= n || n <= 0) return;
