@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(_HERE, "libaicomp_kv.so")
 SYMBOLS = (
     "aicomp_kv_version",
     "aicomp_kv_last_error",
+    "aicomp_kv_set_small_decode_tokens",
     "aicomp_kv_append",
     "aicomp_paged_decode_attn",
     "aicomp_paged_decode_attn_append",
@@ -42,6 +43,8 @@ def _declare(lib: C.CDLL) -> None:
     lib.aicomp_kv_version.argtypes = []
     lib.aicomp_kv_last_error.restype = C.c_char_p
     lib.aicomp_kv_last_error.argtypes = []
+    lib.aicomp_kv_set_small_decode_tokens.restype = C.c_longlong
+    lib.aicomp_kv_set_small_decode_tokens.argtypes = [C.c_longlong]
     lib.aicomp_kv_append.restype = i32
     lib.aicomp_kv_append.argtypes = [vp, vp, i64, i64, vp, vp, vp, i64, i32, i32, i32, i64,
                                      i32, i32, vp, vp, vp]

@@ -61,12 +61,20 @@ static bool streamk_shape(int batch, int hq, int hkv, int d, int bs, int q_dtype
 // one workgroup per (row, KV head, partition) on the grid schedule, without any merge kernel when
 // no row can be longer than 640 tokens (measured on 1 to 16 rows of 512 and 2048 tokens: 5.4-8.5
 // against 9-13 us, 8-15 against 11-17 us).  "Small" is rows x (table width x block size) at or
-// below AICOMP_KV_SMALL_DECODE_TOKENS (default 32768; 0 keeps every automatic call of a supported
-// shape on the balanced schedule).
+// below a process-wide threshold: 32768 by default, or the value of the environment variable
+// AICOMP_KV_SMALL_DECODE_TOKENS when the library first needs it (read once, never again), or what
+// aicomp_kv_set_small_decode_tokens() stored last (0 keeps every automatic call of a supported
+// shape on the balanced schedule).  The sizing helpers and the decode calls read the same word.
+static std::atomic<long long>& small_decode_tokens() {
+    static std::atomic<long long> limit{[] {
+        const char* e = getenv("AICOMP_KV_SMALL_DECODE_TOKENS");
+        return e ? atoll(e) : 32768LL;
+    }()};
+    return limit;
+}
+
 static bool small_call(int64_t rows, int bs, int max_blocks) {
-    long long limit = 32768;
-    if (const char* e = getenv("AICOMP_KV_SMALL_DECODE_TOKENS")) limit = atoll(e);
-    return rows * (int64_t)max_blocks * bs <= limit;
+    return rows * (int64_t)max_blocks * bs <= small_decode_tokens().load(std::memory_order_relaxed);
 }
 
 static int auto_partition(int64_t rows, int hkv, int bs, int max_blocks, bool matrix_shape) {
@@ -96,6 +104,11 @@ extern "C" {
 int aicomp_kv_version(void) { return 100; }
 
 const char* aicomp_kv_last_error(void) { return g_err; }
+
+long long aicomp_kv_set_small_decode_tokens(long long tokens) {
+    std::atomic<long long>& limit = small_decode_tokens();
+    return tokens < 0 ? limit.load(std::memory_order_relaxed) : limit.exchange(tokens, std::memory_order_relaxed);
+}
 
 int aicomp_kv_append(const void* key, const void* value, int64_t kv_token_stride,
                      int64_t kv_head_stride, void* k_pool, void* v_pool,

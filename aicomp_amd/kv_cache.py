@@ -128,16 +128,20 @@ class _PagedLayer:
             call = ops.PreparedDecode(self.k_pool, self.v_pool, self.block_table, self.context_lens, Hq,
                                       query.dtype, scale)
             self._decode[(Hq, query.dtype, scale)] = call
-        if live:
-            self.live_ctx.add_(1)                 # a fill-type kernel: safe inside a captured graph
-            ctx = self.live_ctx.data_ptr()
-        else:
-            # row pos + 1 of the context-length table, by address (a view tensor costs microseconds)
-            ctx = self._ctx_base + (pos + 1) * self._ctx_pitch
         if not query.is_contiguous():
             query = query.contiguous()
+        if live:
+            # the counter moves only once the call's arguments have passed their checks (a rejected
+            # call must leave it where it was); add_ is a fill-type kernel, safe inside a captured graph
+            ctx, ready = self.live_ctx.data_ptr(), self._bump_live
+        else:
+            # row pos + 1 of the context-length table, by address (a view tensor costs microseconds)
+            ctx, ready = self._ctx_base + (pos + 1) * self._ctx_pitch, None
         # [B, Hq, 1, D] has the memory layout of [B, Hq, D]: the call takes the tensors as they are
-        return call.step4d(torch.empty_like(query), query, key, value, group, ctx)
+        return call.step4d(torch.empty_like(query), query, key, value, group, ctx, ready)
+
+    def _bump_live(self) -> None:
+        self.live_ctx.add_(1)
 
     def attend(self, query: torch.Tensor, pos: int, scale: float) -> torch.Tensor:
         """query ``[B, Hq, n, D]`` at positions pos..pos+n (rows already appended)."""
@@ -158,8 +162,8 @@ class _PagedLayer:
                                ctx, self.cu_q_lens, scale, max_q_len=n)
         return out.view(B, n, Hq, D).permute(0, 2, 1, 3)
 
-    def gather(self, end: int, heads: int) -> Tuple[torch.Tensor, torch.Tensor]:
-        """Dense ``[B, heads, end, D]`` copies (heads = Hkv or the expanded count)."""
+    def gather(self, end: int, heads: int, which: str = "kv") -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+        """Dense ``[B, heads, end, D]`` copies (heads = Hkv or the expanded count) of K, V or both."""
         B, bps, bs = self.batch, self.blocks_per_seq, self.block_size
 
         def dense(pool):
@@ -169,13 +173,18 @@ class _PagedLayer:
                 x = x.repeat_interleave(heads // self.kv_heads, dim=1)
             return x.contiguous()
 
-        return dense(self.k_pool), dense(self.v_pool)
+        return (dense(self.k_pool) if "k" in which else None, dense(self.v_pool) if "v" in which else None)
 
 
 class PagedKVView:
     """What ``KVCacheManager.update/get`` hand back in place of the reference's
-    ``cache[:, :, :end, :]`` views: the prefix of one layer's K or V.  It stays
-    paged until a caller asks for a tensor (``contiguous()`` / ``to_dense()``)."""
+    ``cache[:, :, :end, :]`` views (``kv_cache.py:166-170, 172-195``): the prefix
+    ``[B, heads, end, D]`` of one layer's K or V.  It stays paged until a caller touches the
+    data; then it gathers a dense tensor of the pool's current contents (like the reference's
+    view, it shows rows written after it was made) and behaves as that tensor: ``shape``,
+    ``dtype``, ``device``, ``dim()`` and ``size()`` cost nothing; indexing, ``torch.*``
+    functions and every other tensor method (``.float()``, ``.transpose(...)``, ...) run on
+    the gathered copy.  It is read-only: the pools are written by ``update`` alone."""
 
     def __init__(self, layer: _PagedLayer, which: str, end: int, heads: int):
         self._layer, self._which, self.end, self.heads = layer, which, end, heads
@@ -187,11 +196,56 @@ class PagedKVView:
     def size(self, dim: Optional[int] = None):
         return self.shape if dim is None else self.shape[dim]
 
+    def dim(self) -> int:
+        return 4
+
+    ndim = property(dim)
+
+    def numel(self) -> int:
+        return self.shape.numel()
+
+    @property
+    def dtype(self) -> torch.dtype:
+        return self._layer.k_pool.dtype
+
+    @property
+    def device(self) -> torch.device:
+        return self._layer.k_pool.device
+
+    @property
+    def is_cuda(self) -> bool:
+        return self._layer.k_pool.is_cuda
+
     def to_dense(self) -> torch.Tensor:
-        k, v = self._layer.gather(self.end, self.heads)
+        k, v = self._layer.gather(self.end, self.heads, self._which)
         return k if self._which == "k" else v
 
     contiguous = to_dense
+
+    def __len__(self) -> int:
+        return self._layer.batch
+
+    def __getitem__(self, index):
+        return self.to_dense()[index]
+
+    def __setitem__(self, index, value):
+        raise TypeError("a PagedKVView is read-only: rows enter the pools through KVCacheManager.update")
+
+    def __getattr__(self, name):
+        # anything else a tensor offers, on the gathered copy (only reached for names not defined above)
+        if name.startswith("_"):
+            raise AttributeError(name)
+        return getattr(self.to_dense(), name)
+
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        dense = lambda x: x.to_dense() if isinstance(x, PagedKVView) else x
+        args = tuple(type(a)(dense(x) for x in a) if isinstance(a, (list, tuple)) else dense(a) for a in args)
+        kwargs = {k: dense(v) for k, v in (kwargs or {}).items()}
+        return func(*args, **kwargs)
+
+    def __repr__(self) -> str:
+        return f"PagedKVView({self._which}, shape={tuple(self.shape)}, dtype={self.dtype}, device={self.device})"
 
 
 class KVCacheManager:
@@ -410,7 +464,17 @@ class CachedScaledDotProductAttention(nn.Module):
             if self._store is None:
                 raise RuntimeError("device positions start from an ingested prompt: run the prefill first")
             self._store.live_ctx.fill_(self.cache_pos)
+        elif self._device_positions:
+            self._resync_position()
         self._device_positions = on
+
+    def _resync_position(self) -> None:
+        """Leaving device positions: the device counter is the truth (replays advanced it without
+        running Python), so the host position is read back from it - one device-to-host copy,
+        outside any capture.  A caller that forgot ``advance(n)`` therefore cannot end up writing
+        over live tokens."""
+        if self._store is not None and not torch.cuda.is_current_stream_capturing():
+            self.cache_pos = min(int(self._store.live_ctx[0].item()), self.max_seq_len)
 
     def advance(self, steps: int) -> None:
         """Account on the host for decode steps that were replayed from a graph."""
@@ -422,7 +486,7 @@ class CachedScaledDotProductAttention(nn.Module):
     def clear(self) -> None:
         """Reset the write position; the allocation is kept (``kv_cache.py:324-338``)."""
         self.cache_pos = 0
-        self._device_positions = False
+        self._device_positions = False          # the next use_device_positions() starts the counter afresh
 
     def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                 attn_mask: Optional[torch.Tensor] = None, dropout_p: float = 0.0,
@@ -458,15 +522,22 @@ class CachedScaledDotProductAttention(nn.Module):
                 self._group = group
                 self._store = _PagedLayer(B, Hk // group, D, self.max_seq_len, key.dtype, key.device)
             store = self._store
+            if self._device_positions and n != 1:
+                # a prompt chunk while decode positions live on the device: take the position from
+                # the device counter first, then go on with host positions
+                self._resync_position()
+                self._device_positions = False
+                pos = self.cache_pos
             if pos + n > self.max_seq_len:
                 raise RuntimeError(f"cache overflow: position {pos} + {n} new tokens > max_seq_len "
                                    f"{self.max_seq_len}")
             if n == 1 and key.dtype == store.k_pool.dtype:
                 # decode step: append fused into the attention call.  A call that is only being
                 # recorded into a graph executes nothing: the host position stays (see advance()).
+                out = store.decode_step(query, key, value, pos, self._group, scale, live=self._device_positions)
                 if not (self._device_positions and torch.cuda.is_current_stream_capturing()):
-                    self.cache_pos = pos + 1
-                return store.decode_step(query, key, value, pos, self._group, scale, live=self._device_positions)
+                    self.cache_pos = pos + 1      # only after the call was accepted
+                return out
             store.append(key, value, pos, self._group)
         self.cache_pos = pos + n
         # the caller's attn_mask is dropped, as in the reference (kv_cache.py:400-415): decode sees

@@ -118,6 +118,21 @@ def _workspace(device: torch.device, nbytes: int, stream: Optional[int] = None) 
     return buf
 
 
+# bumped whenever the routing threshold changes: sizes cached under an older value are asked for again
+_route_epoch = 0
+
+
+def set_small_decode_tokens(tokens: int) -> int:
+    """Set the library's routing threshold between the two decode schedules (tokens = rows x table
+    width x block size up to which an automatic call takes the grid schedule; 0: always balanced)
+    and return the previous value; a negative value only queries.  Process-wide."""
+    global _route_epoch
+    prev = int(_lib.load().aicomp_kv_set_small_decode_tokens(int(tokens)))
+    if tokens >= 0 and tokens != prev:
+        _route_epoch += 1
+    return prev
+
+
 def decode_partition_size(batch: int, hq: int, hkv: int, d: int, bs: int, max_blocks: int,
                           q_dtype: torch.dtype, kv_dtype: torch.dtype) -> int:
     lib = _lib.load()
@@ -234,13 +249,20 @@ class PreparedDecode:
         self.q_shape = (B, num_q_heads, d)
         self.kv_shape = (B, hkv, d)
         self.context_lens = context_lens
-        self.need = self.lib.aicomp_paged_decode_workspace_bytes(B, num_q_heads, hkv, d, bs, block_table.shape[1],
-                                                                 qd, _dt(k_pool, "pool"), partition_size)
+        self._need_args = (B, num_q_heads, hkv, d, bs, block_table.shape[1], qd, _dt(k_pool, "pool"), partition_size)
+        self._need, self._epoch = self.lib.aicomp_paged_decode_workspace_bytes(*self._need_args), _route_epoch
         # keep the tensors alive; everything below is what the C entry points take
         self._keep = (k_pool, v_pool, block_table, ks, vs)
         self._head = (k_pool.data_ptr(), v_pool.data_ptr(), block_table.data_ptr(), block_table.stride(0))
         self._tail = (B, num_q_heads, hkv, d, bs, block_table.shape[1], nb, float(scale), qd,
                       _dt(k_pool, "pool"), _ptr(ks), _ptr(vs), partition_size)
+
+    @property
+    def need(self) -> int:
+        """Scratch bytes of a call, for the routing threshold in force now."""
+        if self._epoch != _route_epoch:
+            self._need, self._epoch = self.lib.aicomp_paged_decode_workspace_bytes(*self._need_args), _route_epoch
+        return self._need
 
     def __call__(self, out: torch.Tensor, query: torch.Tensor, new_key: Optional[torch.Tensor] = None,
                  new_value: Optional[torch.Tensor] = None,
@@ -271,12 +293,14 @@ class PreparedDecode:
         return out
 
     def step4d(self, out: torch.Tensor, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
-               group: int, context_lens) -> torch.Tensor:
+               group: int, context_lens, ready=None) -> torch.Tensor:
         """The fused append + decode call on the operator's own tensors: ``query`` / ``out``
         ``[B, Hq, 1, D]`` contiguous, ``key`` / ``value`` ``[B, H, 1, D]`` with H = Hkv or
         Hkv * group (heads repeated ``group`` times, as HF's ``repeat_kv`` leaves them: every
         group-th head is read).  No view tensors are made: the strides go to the library as they
-        are.  ``context_lens`` is an int32 ``[B]`` tensor on the device, or its device address."""
+        are.  ``context_lens`` is an int32 ``[B]`` tensor on the device, or its device address.
+        ``ready``, if given, is called once the arguments have passed every check, right before
+        the launch (for work that must not happen for a rejected call)."""
         B, Hq, D = self.q_shape
         hkv = self.kv_shape[1]
         H = key.shape[1]
@@ -293,6 +317,8 @@ class PreparedDecode:
         stream = _current_stream(self.device)
         ws = _workspace(self.device, self.need, stream)
         ws_ptr, ws_bytes = (None, 0) if ws is None else (ws.data_ptr(), ws.numel())
+        if ready is not None:
+            ready()
         rc = self.lib.aicomp_paged_decode_attn_append(
             out.data_ptr(), query.data_ptr(), key.data_ptr(), value.data_ptr(),
             key.stride(0), key.stride(1) * hstep, *self._head,

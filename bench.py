@@ -41,6 +41,38 @@ def measured_traffic_bytes():
         return None
 
 
+def profiled_prefill_cycles():
+    """Shader cycles of one prefill launch of the chunked-prefill shape, from the kept rocprofv3
+    counter summary (SQ_BUSY_CYCLES / 32 shader engines); None if the summary is missing."""
+    import re
+    try:
+        with open(os.path.join(ROOT, "profiles", "prefill_chunked_prefill_mixed.md")) as f:
+            m = re.search(r"([0-9]+) cycles per launch", f.read())
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
+def settled_back_to_back(fn, reps=50, settle_s=0.03):
+    """Average duration of `reps` launches of fn queued back to back between two events, after
+    `settle_s` of untimed launches (an idle GPU's clock takes that long to ramp up)."""
+    import torch
+    fn()
+    torch.cuda.synchronize()
+    tw = time.perf_counter()
+    while time.perf_counter() - tw < settle_s:
+        for _ in range(8):
+            fn()
+        torch.cuda.synchronize()
+    p0, p1 = _events(2)
+    p0.record()
+    for _ in range(reps):
+        fn()
+    p1.record()
+    torch.cuda.synchronize()
+    return p0.elapsed_time(p1) / reps * 1e-3
+
+
 def _events(n):
     import torch
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
@@ -72,45 +104,60 @@ def run_decode_config(name, steps, warmup, dev):
     nk_dec = w.new_key[t0_dec:].contiguous()
     nv_dec = w.new_value[t0_dec:].contiguous()
 
-    def step(ev=None):
+    # A model step walks one K/V pool per layer, so no call finds its pool in a cache the previous
+    # call filled.  The timed loop does the same: it cycles over several pools ("layers": same
+    # tables and lengths, separate allocations), enough of them that a pool has been pushed out of
+    # the 256 MB memory-side cache and the L2s by the time its turn comes again.
+    pool_bytes = 2 * w.k_pool.numel() * w.k_pool.element_size()
+    n_pools = int(min(32, max(3, -(-(1 << 30) // pool_bytes))))
+    pools = [(w.k_pool, w.v_pool)] + [(w.k_pool.clone(), w.v_pool.clone()) for _ in range(n_pools - 1)]
+
+    def step(i=0, ev=None):
+        kp, vp = pools[i % len(pools)]
         if ev: ev[0].record()
         if npre:
             # mixed step: scatter every new row (chunks and decode tokens), prefill, decode
-            ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping, w.k_scale, w.v_scale)
+            ops.kv_append(w.new_key, w.new_value, kp, vp, w.slot_mapping, w.k_scale, w.v_scale)
             if ev: ev[1].record()
-            ops.paged_prefill_attn(outp, qp, w.k_pool, w.v_pool, btp, clp, cup, w.scale, max_q_len=max_q)
+            ops.paged_prefill_attn(outp, qp, kp, vp, btp, clp, cup, w.scale, max_q_len=max_q)
             if ev: ev[2].record()
-            ops.paged_decode_attn(outd, qd, w.k_pool, w.v_pool, btd, cld, w.scale, w.k_scale, w.v_scale)
+            ops.paged_decode_attn(outd, qd, kp, vp, btd, cld, w.scale, w.k_scale, w.v_scale)
         else:
             # decode step: the append of the 1-token-per-sequence rows is fused into the call
             if ev: ev[1].record()
-            ops.paged_decode_attn(outd, qd, w.k_pool, w.v_pool, btd, cld, w.scale, w.k_scale, w.v_scale,
+            ops.paged_decode_attn(outd, qd, kp, vp, btd, cld, w.scale, w.k_scale, w.v_scale,
                                   new_key=nk_dec, new_value=nv_dec)
         if ev: ev[3].record()
 
     def append_only():
         ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping, w.k_scale, w.v_scale)
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    # Two HIP events bracket the timed region on the launch stream: with the steps queued back to
-    # back their distance / K is the average duration of a step's launches.  A step that has
-    # several phases (append, prefill, decode) also carries events between the phases, but only on
-    # ten of the steps: an event costs a few microseconds of stream time.
-    stride = max(1, steps // 10)
-    evs = {i: _events(4) for i in range(0, steps, stride)} if npre else {}
-    r_begin, r_end = _events(2)
-    t0 = time.perf_counter()
-    r_begin.record()
-    for i in range(steps):
-        step(evs.get(i))
-    r_end.record()
-    t_enqueue = time.perf_counter() - t0
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    region = r_begin.elapsed_time(r_end) / steps * 1e-3     # seconds per step, device time line
-    evs = list(evs.values())
+    def timed_loop(rotate):
+        """K steps queued back to back between two HIP events on the launch stream: their distance
+        / K is the average duration of a step's launches.  A step that has several phases (append,
+        prefill, decode) also carries events between the phases, but only on ten of the steps: an
+        event costs a few microseconds of stream time."""
+        for i in range(warmup):
+            step(i if rotate else 0)
+        torch.cuda.synchronize()
+        stride = max(1, steps // 10)
+        evs = {i: _events(4) for i in range(0, steps, stride)} if npre else {}
+        r_begin, r_end = _events(2)
+        t0 = time.perf_counter()
+        r_begin.record()
+        for i in range(steps):
+            step(i if rotate else 0, evs.get(i))
+        r_end.record()
+        t_enqueue = time.perf_counter() - t0
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        region = r_begin.elapsed_time(r_end) / steps * 1e-3     # seconds per step, device time line
+        return wall, t_enqueue, region, list(evs.values())
+
+    # the same loop over one pool (every step re-reads what the previous one read): kept beside
+    # the rotating figure, which is the one the headline uses
+    wall_1, _, region_1, evs_1 = timed_loop(rotate=False)
+    wall, t_enqueue, region, evs = timed_loop(rotate=True)
     # the stand-alone append kernel, timed on its own: 20 launches between two events, queued
     # behind ~1 ms of filler work so that the host's launch rate does not enter the figure
     for _ in range(3):
@@ -151,7 +198,7 @@ def run_decode_config(name, steps, warmup, dev):
     # the same decode step recorded into a HIP graph (ten calls per graph, so that the graph's own
     # launch cost is shared) and replayed: no host launch cost per step (the library allocates
     # nothing and clears nothing, the scratch is passed in)
-    GRAPH_CALLS = 10
+    GRAPH_CALLS = len(pools) * -(-10 // len(pools))       # whole turns of the pool cycle
     t_graph = None
     if not npre:
         try:
@@ -160,8 +207,8 @@ def run_decode_config(name, steps, warmup, dev):
             ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                for _ in range(GRAPH_CALLS):
-                    ops.paged_decode_attn(outd, qd, w.k_pool, w.v_pool, btd, cld, w.scale, w.k_scale, w.v_scale,
+                for i in range(GRAPH_CALLS):
+                    ops.paged_decode_attn(outd, qd, *pools[i % len(pools)], btd, cld, w.scale, w.k_scale, w.v_scale,
                                           new_key=nk_dec, new_value=nv_dec, workspace=ws)
             for _ in range(3):
                 graph.replay()
@@ -176,36 +223,30 @@ def run_decode_config(name, steps, warmup, dev):
         except Exception as e:                              # a bench figure, not a requirement
             print(f"graph replay not measured for {name}: {e}", file=sys.stderr)
     t_app = a0.elapsed_time(a1) / 20 * 1e-3
-    t_pre_in_step = statistics.mean(e[1].elapsed_time(e[2]) for e in evs) * 1e-3 if npre else 0.0
-    t_pre = 0.0
+    t_pre = statistics.mean(e[1].elapsed_time(e[2]) for e in evs) * 1e-3 if npre else 0.0
+    t_pre_b2b = 0.0
     if npre:
-        # The prefill kernel's average launch duration: launches queued back to back between two
-        # events, after ~30 ms of untimed ones (the first launches after an idle gap run 10-15 %
-        # slower while the clock ramps up, and a pair of events around a single launch inside the
-        # mixed step adds their own stream time; that figure is kept as prefill_in_step_us).
-        pre = lambda: ops.paged_prefill_attn(outp, qp, w.k_pool, w.v_pool, btp, clp, cup, w.scale, max_q_len=max_q)
-        tw = time.perf_counter()
-        while time.perf_counter() - tw < 0.03:
-            for _ in range(8):
-                pre()
-            torch.cuda.synchronize()
-        p0, p1 = _events(2)
-        p0.record()
-        for _ in range(50):
-            pre()
-        p1.record()
-        torch.cuda.synchronize()
-        t_pre = p0.elapsed_time(p1) / 50 * 1e-3
+        # prefill_us and prefill_roofline describe the launch inside the mixed step (events around it,
+        # pools rotating).  Beside it, under its own key: launches queued back to back between two
+        # events after ~30 ms of untimed ones (the first launches after an idle gap run 10-15 %
+        # slower while the clock ramps up; this is the protocol of `--only prefill`, whose
+        # rocprofv3 summary under profiles/ it can be compared with).
+        t_pre_b2b = settled_back_to_back(
+            lambda: ops.paged_prefill_attn(outp, qp, w.k_pool, w.v_pool, btp, clp, cup, w.scale, max_q_len=max_q))
     # a pure decode step is one call (main + merge kernel): its average duration is the region's
     t_dec = statistics.mean(e[2].elapsed_time(e[3]) for e in evs) * 1e-3 if npre else region
-    # A tiny step is bound by the host's launch rate, not by the GPU: the eager loop then measures
-    # Python, and the call's duration on the GPU is what it takes inside the replayed graph.
+    t_dec_1 = statistics.mean(e[2].elapsed_time(e[3]) for e in evs_1) * 1e-3 if npre else region_1
+    # A tiny step is bound by the host's launch rate, not by the GPU: the eager figures then measure
+    # Python.  They stay what they are (decode_us is what the eager operator path delivers); the
+    # call's duration on the GPU, inside the replayed graph, is reported beside them.
     host_bound = (not npre) and t_graph is not None and t_enqueue / steps > 0.9 * region
-    t_dec_eager = t_dec
-    if host_bound:
-        t_dec = t_graph
+    mb = btd.shape[1]
+    routed_small = (S - npre) * mb * w.shape.block_size <= ops.set_small_decode_tokens(-1)
     res = {
-        "workload": name, "ms_per_step": wall / steps * 1e3,
+        "workload": name, "ms_per_step": wall / steps * 1e3, "pools_in_rotation": len(pools),
+        "single_pool": {"ms_per_step": wall_1 / steps * 1e3, "decode_us": t_dec_1 * 1e6,
+                        "decode_frac_hbm_peak": w.decode_kv_bytes() / t_dec_1 / 1e9 / HBM_PEAK_GBS,
+                        "note": "the same loop re-reading one pool every step"},
         "host_enqueue_ms_per_step": t_enqueue / steps * 1e3,
         "append_us": t_app * 1e6, "append_bytes": w.append_bytes(),
         "append_GBs": w.append_bytes() / t_app / 1e9,
@@ -217,28 +258,40 @@ def run_decode_config(name, steps, warmup, dev):
         "decode_tokens_per_s": (S - npre) / t_dec,
         "decode_cold_us": t_cold * 1e6, "decode_cold_GBs": w.decode_kv_bytes() / t_cold / 1e9,
         "decode_graph_replay_us": None if t_graph is None else t_graph * 1e6,
-        "decode_eager_us": t_dec_eager * 1e6, "decode_timed_in_graph": bool(host_bound),
+        "decode_graph_replay_GBs": None if t_graph is None else w.decode_kv_bytes() / t_graph / 1e9,
+        "host_bound": bool(host_bound),
         "partition_size": ops.decode_partition_size(S - npre, w.shape.num_q_heads, w.shape.num_kv_heads,
                                                     w.shape.head_dim, w.shape.block_size, btd.shape[1],
                                                     qd.dtype, w.k_pool.dtype),
         "kv_dtype": str(w.k_pool.dtype).replace("torch.", ""),
     }
     mfma_shape = (w.shape.head_dim in (64, 128) and w.shape.block_size == 16 and qd.dtype in (torch.bfloat16, torch.float16))
-    balanced = mfma_shape and (S - npre) <= 1024
+    balanced = mfma_shape and (S - npre) <= 1024 and not routed_small        # the library's own routing rule
+    merge = "" if res["partition_size"] >= mb * w.shape.block_size else " + split_reduce_kernel"
     res["roofline"] = {
         "kernel": ("streamk_decode_kernel + streamk_reduce_kernel" if balanced else
-                   "paged_decode_mfma_kernel + split_reduce_kernel" if mfma_shape else
-                   "paged_attn_generic_kernel + split_reduce_kernel"),
+                   "paged_decode_mfma_kernel" + merge if mfma_shape else
+                   "paged_attn_generic_kernel" + merge),
         "bound": "hbm", "achieved": res["decode_GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": res["decode_frac_hbm_peak"], "algorithmic_bytes": res["decode_bytes"], "avg_launch_us": res["decode_us"]}
     if npre:
-        res.update({"prefill_us": t_pre * 1e6, "prefill_in_step_us": t_pre_in_step * 1e6, "prefill_flops": w.prefill_flops(),
+        cyc = profiled_prefill_cycles()
+        res.update({"prefill_us": t_pre * 1e6, "prefill_back_to_back_us": t_pre_b2b * 1e6,
+                    "prefill_flops": w.prefill_flops(),
                     "prefill_TFLOPs": w.prefill_flops() / t_pre / 1e12,
-                    "prefill_frac_mfma_peak": w.prefill_flops() / t_pre / 1e12 / MFMA_BF16_PEAK_TFLOPS})
+                    "prefill_frac_mfma_peak": w.prefill_flops() / t_pre / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                    "prefill_back_to_back_frac_mfma_peak": w.prefill_flops() / t_pre_b2b / 1e12 / MFMA_BF16_PEAK_TFLOPS})
         res["prefill_roofline"] = {
             "kernel": "paged_prefill_mfma_kernel", "bound": "mfma", "achieved": res["prefill_TFLOPs"],
             "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": res["prefill_frac_mfma_peak"],
-            "algorithmic_flop": res["prefill_flops"], "avg_launch_us": res["prefill_us"]}
+            "algorithmic_flop": res["prefill_flops"], "avg_launch_us": res["prefill_us"],
+            "timed": "the launch inside the mixed step, between two events",
+            # the launch's length in shader cycles does not depend on the clock the part happens to
+            # hold (profiles/prefill_chunked_prefill_mixed.md, SQ_BUSY_CYCLES per shader engine), so
+            # cycles / duration is the clock a timing was taken at; the peak assumes 2.4 GHz
+            "cycles_per_launch": cyc,
+            "clock_GHz_in_step": None if cyc is None else cyc / (t_pre * 1e6) / 1e3,
+            "clock_GHz_back_to_back": None if cyc is None else cyc / (t_pre_b2b * 1e6) / 1e3}
     return res, w
 
 
@@ -457,27 +510,44 @@ def rope_case(w, dev):
     return fn, nbytes
 
 
-def profile_target(which, steps, warmup, dev):
+def profile_target(which, steps, warmup, dev, settle_ms=30.0):
     """Launch one kernel of the path repeatedly, for rocprofv3 (--kernel-trace / --pmc).
-    "copy" is a plain device copy of exactly 1 GiB: the counter calibration."""
+    "copy" is a plain device copy of exactly 1 GiB: the counter calibration.
+
+    The launches follow the protocol of the bench's back-to-back timings: `warmup` untimed
+    launches, then untimed launches for `settle_ms` more (the clock of an idle part takes about
+    that long to ramp up), then `steps` launches queued back to back; a summary averages the last
+    `steps` dispatches of the trace.  Counter passes use --settle-ms 0 (they serialise launches)."""
     import torch
     from aicomp_amd import ops, workloads
+
+    def drive(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        settled = 0
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < settle_ms:
+            for _ in range(8):
+                fn()
+            settled += 8
+            torch.cuda.synchronize()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return f"{warmup} + {settled} untimed launches, then {steps} back to back"
     if which == "copy":
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
-        for _ in range(warmup + steps):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        print(f"copy: {steps + warmup} launches of {src.numel()} bytes read + {dst.numel()} bytes written")
+        how = drive(lambda: dst.copy_(src))
+        print(f"copy: {how}; {src.numel()} bytes read + {dst.numel()} bytes written per launch")
         return
     if which == "sample":
         g = torch.Generator(device=dev).manual_seed(0)
         logits = torch.randn(64, 128256, device=dev, generator=g) * 2.5
         u = torch.rand(64, device=dev, generator=g)
-        for _ in range(warmup + steps):
-            ops.sample_tokens(logits, 0.8, 50, 0.9, uniforms=u)
-        torch.cuda.synchronize()
-        print(f"sample: {steps + warmup} launches over [64, 128256] fp32 logits, temperature 0.8, top-k 50, top-p 0.9")
+        how = drive(lambda: ops.sample_tokens(logits, 0.8, 50, 0.9, uniforms=u))
+        print(f"sample: {how}, over [64, 128256] fp32 logits, temperature 0.8, top-k 50, top-p 0.9")
         return
     if which == "prefill_long":
         # one fresh prompt of 8192 tokens at the Llama-3-8B head shape (a row of prefill_other_shapes)
@@ -492,10 +562,8 @@ def profile_target(which, steps, warmup, dev):
         o = torch.empty_like(q)
         cl = torch.full((1,), n, dtype=torch.int32, device=dev)
         cu = torch.tensor([0, n], dtype=torch.int32, device=dev)
-        for _ in range(warmup + steps):
-            ops.paged_prefill_attn(o, q, k, v, table, cl, cu, 1 / math.sqrt(d), max_q_len=n)
-        torch.cuda.synchronize()
-        print(f"prefill_long: {steps + warmup} launches, {4 * hq * d * (n * (n + 1) // 2)} algorithmic flop per launch")
+        how = drive(lambda: ops.paged_prefill_attn(o, q, k, v, table, cl, cu, 1 / math.sqrt(d), max_q_len=n))
+        print(f"prefill_long: {how}, {4 * hq * d * (n * (n + 1) // 2)} algorithmic flop per launch")
         return
     name = {"decode": "llama3_8b_decode", "append": "chunked_prefill_mixed", "prefill": "chunked_prefill_mixed",
             "decode_fp8": "llama3_70b_decode_fp8", "decode_long": "long_context_skewed",
@@ -523,10 +591,23 @@ def profile_target(which, steps, warmup, dev):
         mq = max(w.new_list[:npre])
         fn = lambda: ops.paged_prefill_attn(out, q, w.k_pool, w.v_pool, bt, cl, cu, w.scale, max_q_len=mq)
         info = f"{w.prefill_flops()} algorithmic flop per launch"
-    for _ in range(warmup + steps):
-        fn()
-    torch.cuda.synchronize()
-    print(f"{which} ({name}): {steps + warmup} launches, {info}")
+    how = drive(fn)
+    print(f"{which} ({name}): {how}, {info}")
+
+
+def host_threads():
+    """torch.set_num_threads(<the host cores this process may use>), called explicitly: os.cpu_count(),
+    held to the share the environment grants where it states one (OMP_NUM_THREADS).  Returns the
+    thread count torch reports afterwards."""
+    import torch
+    n = os.cpu_count() or 1
+    try:
+        n = max(1, min(n, int(os.environ.get("OMP_NUM_THREADS", n))))
+    except ValueError:
+        pass
+    if torch.get_num_threads() != n:
+        torch.set_num_threads(n)
+    return torch.get_num_threads()
 
 
 def cpu_baseline(w, budget_s=20.0):
@@ -534,7 +615,7 @@ def cpu_baseline(w, budget_s=20.0):
     oracle/contiguous_ref.py, timed on the host cores over a bounded sample of the batch."""
     import torch
     from oracle import contiguous_ref as cref
-    threads = torch.get_num_threads()
+    threads = host_threads()
     npre = w.num_prefill_seqs
     q = w.query[int(w.cu_q_lens[npre]):].cpu()
     bt = w.block_table[npre:].cpu()
@@ -556,7 +637,7 @@ def cpu_baseline(w, budget_s=20.0):
     per_seq = t1 / n
     nseq = int(max(1, min(B, budget_s / (6 * per_seq))))
     reps = int(max(3, min(10, budget_s / (per_seq * nseq) - 3)))
-    for _ in range(2):
+    for _ in range(3):
         run(nseq)
     ts = sorted(run(nseq) for _ in range(reps))
     med = ts[len(ts) // 2]
@@ -576,7 +657,7 @@ def cpu_baseline(w, budget_s=20.0):
             "tokens_per_s": nseq / med,
             "sample": f"first {nseq} of {B} sequences of the same batch, decode attention only "
                       f"(gather blocks -> repeat_kv -> contiguous -> torch SDPA, {str(q.dtype).replace('torch.', '')}), "
-                      f"2 warmups, median of {reps}; {med * 1e3:.1f} ms per pass; "
+                      f"3 warmups, median of {reps}; {med * 1e3:.1f} ms per pass; "
                       f"cpu '{model}', os.cpu_count()={os.cpu_count()}, torch threads={threads}"}
 
 
@@ -585,6 +666,7 @@ def cpu_prefill_baseline(w):
     oracle/contiguous_ref.py, timed on the host cores for the first chunk of the workload."""
     import torch
     from oracle import contiguous_ref as cref
+    host_threads()
     n, L = w.new_list[0], w.ctx_list[0]
     q = w.query[: n].cpu()
     bt = w.block_table[0].cpu()
@@ -614,6 +696,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     ap.add_argument("--only", choices=["decode", "append", "copy", "prefill", "prefill_long", "decode_fp8", "decode_long", "decode_d64", "rope", "sample"],
                     help="profiling target: launch just this kernel --steps times (no JSON line)")
+    ap.add_argument("--settle-ms", type=float, default=30.0,
+                    help="with --only: untimed launches for this long before the timed ones")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on one GPU only (asked for --gpus {args.gpus}); "
@@ -629,7 +713,7 @@ def main():
     dev = torch.device("cuda:0")
 
     if args.only:
-        profile_target(args.only, args.steps, args.warmup, dev)
+        profile_target(args.only, args.steps, args.warmup, dev, args.settle_ms)
         return
     main_res, w = run_decode_config("llama3_8b_decode", args.steps, args.warmup, dev)
     s = w.shape
@@ -643,7 +727,8 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "llama3_8b_decode: batch 64, 32 query / 8 KV heads, head_dim 128, "
                                "block 16, context uniform [512,4096] seed 0, bf16; step = KV append "
-                               "of 64 rows + paged decode attention (one fused call)",
+                               "of 64 rows + paged decode attention (one fused call); consecutive steps "
+                               "run over different K/V pools, as the layers of a model do",
                    "batch": s.batch, "partition_size": main_res["partition_size"],
                    "kv_bytes_per_step": main_res["decode_bytes"]},
         "tokens_per_s": s.batch / (main_res["ms_per_step"] * 1e-3),
@@ -657,6 +742,8 @@ def main():
         "append": {"us": main_res["append_us"], "GB/s": main_res["append_GBs"],
                    "bytes": main_res["append_bytes"]},
         "decode_graph_replay_us": main_res["decode_graph_replay_us"],
+        "pools_in_rotation": main_res["pools_in_rotation"],
+        "single_pool": main_res["single_pool"],
         "decode_cold": {"us": main_res["decode_cold_us"], "GB/s": main_res["decode_cold_GBs"],
                         "note": "decode call timed right after 1 GiB of unrelated writes"},
         "device": device_info(),

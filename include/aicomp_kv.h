@@ -53,6 +53,21 @@ int aicomp_kv_version(void);
 const char* aicomp_kv_last_error(void);
 
 /*
+ * Routing threshold of automatic decode calls (partition_size 0), in tokens: a call with
+ * batch * max_blocks_per_seq * block_size at or below it takes the grid schedule (see
+ * aicomp_paged_decode_attn), a larger one the balanced schedule; 0 sends every supported shape
+ * to the balanced schedule.  Process-wide; the initial value is 32768, or the value of the
+ * environment variable AICOMP_KV_SMALL_DECODE_TOKENS at the library's first use of it (the
+ * environment is read once, never per call).  Stores `tokens` and returns the previous value; a
+ * negative `tokens` only queries.  aicomp_paged_decode_workspace_bytes and
+ * aicomp_paged_decode_partition_size answer for the value current at their call, so a caller
+ * that changes the threshold asks them again before reusing a cached size.  No counterpart in
+ * the reference (which has a single torch call per step, kv_cache.py:397-403); it exists so
+ * that a host can pin the schedule without touching the environment.
+ */
+long long aicomp_kv_set_small_decode_tokens(long long tokens);
+
+/*
  * KV append: scatter T new rows into the pools by slot_mapping.
  * Replaces  key_cache[:, :, position:end_position, :] = new_k   (kv_cache.py:159-160)
  * and       self.cache_k[:, :, self.cache_pos:end_pos, :] = key (kv_cache.py:387-388).
@@ -105,9 +120,8 @@ int aicomp_kv_append(const void* key, const void* value,
  *                   number of 32-token tiles); a multiple of block_size otherwise.
  *                   Split work is merged by a second kernel from partial
  *                   (max, sum, output) triples.  With 0, a call over few short rows
- *                   (batch * max_blocks_per_seq * block_size at or below the value of
- *                   the environment variable AICOMP_KV_SMALL_DECODE_TOKENS, default
- *                   32768; read at every call) runs one workgroup per (row, KV head,
+ *                   (batch * max_blocks_per_seq * block_size at or below the process-wide
+ *                   threshold of aicomp_kv_set_small_decode_tokens(), default 32768) runs one workgroup per (row, KV head,
  *                   256-token partition) instead, and no merge kernel at all when
  *                   max_blocks_per_seq * block_size <= 640: such a call is bound by
  *                   launch and memory latency, not by bandwidth.  The result is the

@@ -181,6 +181,15 @@ def gather_context(pool: np.ndarray, block_table_row: Sequence[int], length: int
     return out
 
 
+def gather_context_fast(pool: np.ndarray, block_table_row: Sequence[int], length: int) -> np.ndarray:
+    """``gather_context`` as one fancy-indexing expression, for full-size batches (tens of
+    thousands of tokens per sequence); checked element for element against the token loop above."""
+    bs = pool.shape[2]
+    t = np.arange(length)
+    blk = np.asarray(block_table_row, dtype=np.int64)[t // bs]
+    return np.ascontiguousarray(pool[blk, :, t % bs, :])
+
+
 def repeat_kv_index(num_q_heads: int, num_kv_heads: int) -> np.ndarray:
     """KV head read by each query head (modeling_llama.py:268-277)."""
     g = num_q_heads // num_kv_heads
@@ -286,10 +295,12 @@ def paged_decode_attn(
     kv_dtype: str = "f32",
     k_scale: Optional[np.ndarray] = None,
     v_scale: Optional[np.ndarray] = None,
+    gather=gather_context,
 ) -> np.ndarray:
     """query [B, Hq, D] raw -> float64 [B, Hq, D].  One new token per sequence.
 
-    A sequence with context length 0 yields zeros (nothing to attend to).
+    A sequence with context length 0 yields zeros (nothing to attend to).  ``gather`` is the
+    routine that rebuilds a sequence's contiguous prefix (the token loop, or its vectorised twin).
     """
     B, hq, d = query.shape
     out = np.zeros((B, hq, d), dtype=np.float64)
@@ -298,8 +309,8 @@ def paged_decode_attn(
         L = int(context_lens[b])
         if L == 0:
             continue
-        k = decode_elements(gather_context(k_pool, block_table[b], L), kv_dtype)
-        v = decode_elements(gather_context(v_pool, block_table[b], L), kv_dtype)
+        k = decode_elements(gather(k_pool, block_table[b], L), kv_dtype)
+        v = decode_elements(gather(v_pool, block_table[b], L), kv_dtype)
         if k_scale is not None:
             k = k * np.asarray(k_scale, dtype=np.float32).astype(np.float64)[None, :, None]
         if v_scale is not None:
@@ -320,6 +331,7 @@ def paged_prefill_attn(
     kv_dtype: str = "f32",
     k_scale: Optional[np.ndarray] = None,
     v_scale: Optional[np.ndarray] = None,
+    gather=gather_context,
 ) -> np.ndarray:
     """query [T, Hq, D] raw (chunks concatenated) -> float64 [T, Hq, D].
 
@@ -335,8 +347,8 @@ def paged_prefill_attn(
         L = int(context_lens[s])
         if n == 0:
             continue
-        k = decode_elements(gather_context(k_pool, block_table[s], L), kv_dtype)
-        v = decode_elements(gather_context(v_pool, block_table[s], L), kv_dtype)
+        k = decode_elements(gather(k_pool, block_table[s], L), kv_dtype)
+        v = decode_elements(gather(v_pool, block_table[s], L), kv_dtype)
         if k_scale is not None:
             k = k * np.asarray(k_scale, dtype=np.float32).astype(np.float64)[None, :, None]
         if v_scale is not None:

@@ -69,3 +69,27 @@ def test_prefill_kernel_waits_for_its_tile_loads_before_the_step_barrier():
     first_barrier = step.index("__syncthreads()")
     before = re.sub(r"\s+", " ", step[:first_barrier]).strip()
     assert before.endswith("if constexpr (DMA) { __builtin_amdgcn_s_waitcnt(0x0F70);"), before[-200:]
+
+
+def test_routing_threshold_is_one_word_shared_by_sizing_and_calls():
+    """The small-call threshold is process state behind a setter (not an environment lookup per
+    call): set returns the previous value, a negative argument only queries, and the sizing helpers
+    answer for the value in force."""
+    from aicomp_amd import ops
+    lib = _lib.load()
+    prev = lib.aicomp_kv_set_small_decode_tokens(-1)
+    try:
+        assert lib.aicomp_kv_set_small_decode_tokens(0) == prev
+        assert lib.aicomp_kv_set_small_decode_tokens(-5) == 0
+        args = (2, 32, 8, 128, 16, 40, _lib.BF16, _lib.BF16)          # 2 rows x 640 tokens: a small call
+        balanced = lib.aicomp_paged_decode_workspace_bytes(*args, 0)
+        assert balanced > 0                                            # balanced schedule: always a merge
+        assert lib.aicomp_kv_set_small_decode_tokens(32768) == 0
+        assert lib.aicomp_paged_decode_workspace_bytes(*args, 0) == 0  # whole rows on the grid schedule
+        assert lib.aicomp_paged_decode_partition_size(*args) == 640
+        # the Python wrapper bumps an epoch so that prepared calls ask for their size again
+        e0 = ops._route_epoch
+        assert ops.set_small_decode_tokens(0) == 32768 and ops._route_epoch == e0 + 1
+        assert ops.set_small_decode_tokens(0) == 0 and ops._route_epoch == e0 + 1
+    finally:
+        lib.aicomp_kv_set_small_decode_tokens(prev)

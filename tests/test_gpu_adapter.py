@@ -208,3 +208,63 @@ def test_manager_mode_decode_is_one_fused_call_and_equals_internal_mode(device):
         mgr.decode_step(7, mk(1, hq), mk(1, hkv), mk(1, hkv), 0, 0.1)
     with pytest.raises(ValueError):
         mgr.decode_step(0, mk(1, hq), mk(1, hkv), mk(1, hkv), 128, 0.1)
+
+
+def test_manager_views_behave_like_the_reference_tensor_views(device):
+    """``update`` / ``get`` return the prefix ``cache[:, :, :end, :]`` (kv_cache.py:166-170, 172-195).
+    The paged store's stand-in offers the same tensor surface: shape, dtype, device, indexing, torch
+    functions and tensor methods, all equal to the dense prefix a contiguous cache would hold."""
+    B, hq, g, d, n = 2, 8, 4, 64, 37
+    mgr = akv.KVCacheManager(1, B, 128, hq, d, torch.bfloat16, torch.device(device), num_kv_heads=hq // g)
+    mgr.allocate(B)
+    torch.manual_seed(5)
+    k = torch.randn(B, hq // g, n, d).to(torch.bfloat16).repeat_interleave(g, 1).to(device)
+    v = torch.randn(B, hq // g, n, d).to(torch.bfloat16).repeat_interleave(g, 1).to(device)
+    kv, vv = mgr.update(0, k, v)
+    assert kv.shape == (B, hq, n, d) and kv.size(2) == n and kv.dim() == 4 and kv.ndim == 4 and len(kv) == B
+    assert kv.dtype == torch.bfloat16 and kv.device == k.device and kv.is_cuda and kv.numel() == k.numel()
+    eq = lambda a, b: torch.equal(a.view(torch.int16) if a.dtype == torch.bfloat16 else a, b.view(torch.int16) if b.dtype == torch.bfloat16 else b)
+    assert eq(kv.contiguous(), k) and eq(vv.to_dense(), v)
+    assert eq(kv[:, :, -1], k[:, :, -1]) and eq(vv[1, 3, 5:9], v[1, 3, 5:9])          # indexing
+    assert eq(torch.cat([kv, vv], dim=2), torch.cat([k, v], dim=2))                    # torch functions
+    assert torch.equal(torch.matmul(kv.float(), vv.float().transpose(-1, -2)), torch.matmul(k.float(), v.float().transpose(-1, -2)))
+    assert eq(kv.transpose(1, 2), k.transpose(1, 2)) and float(kv.float().sum()) == float(k.float().sum())
+    assert "PagedKVView" in repr(kv)
+    with pytest.raises(TypeError):
+        kv[0] = 0
+    # like the reference's view, a view made earlier shows rows written later inside its range
+    k2 = torch.randn(B, hq // g, 1, d).to(torch.bfloat16).repeat_interleave(g, 1).to(device)
+    mgr.update(0, k2, k2, position=3)
+    assert eq(kv[:, :, 3:4], k2)
+    got_k, got_v = mgr.get(0)
+    assert got_k.shape == (B, hq, n, d) and eq(got_v[:, :, 3:4], k2)
+
+
+def test_device_positions_survive_a_rejected_call_and_a_forgotten_advance(device):
+    """Device-side positions: a call that fails its argument checks moves neither the device counter
+    nor the host position, and leaving the mode takes the position from the device, so decode steps
+    that were never accounted for with ``advance`` cannot be overwritten by the next prompt chunk."""
+    B, hq, g, d = 2, 8, 4, 64
+    op = akv.CachedScaledDotProductAttention(0, 256, num_kv_groups=g)
+    op.enable()
+    mk = lambda n, h=hq: torch.randn(B, h, n, d).to(torch.bfloat16).to(device)
+    op(mk(20), mk(20), mk(20), is_causal=True)
+    op.use_device_positions()
+    with pytest.raises(RuntimeError):
+        op(mk(1), mk(1, hq + 1), mk(1, hq + 1))                     # wrong head count: rejected
+    assert op.cache_pos == 20 and int(op._store.live_ctx[0]) == 20
+    for _ in range(3):
+        op(mk(1), mk(1), mk(1))
+    assert op.cache_pos == 23 and int(op._store.live_ctx[0]) == 23
+    op.cache_pos = 21                                               # as if two replays were never advance()d
+    op.use_device_positions(False)
+    assert op.cache_pos == 23
+    op.use_device_positions()
+    op(mk(1), mk(1), mk(1))
+    op.cache_pos = 20                                               # stale again, then a prompt chunk arrives
+    before = op._store.k_pool.clone()
+    op(mk(5), mk(5), mk(5), is_causal=True)
+    assert op.cache_pos == 29 and not op._device_positions
+    used = op._store.slot_table[:, :24].reshape(-1)
+    flat = lambda p: p.permute(0, 2, 1, 3).reshape(-1, p.shape[1], p.shape[3])
+    assert torch.equal(flat(op._store.k_pool)[used].view(torch.int16), flat(before)[used].view(torch.int16))

@@ -458,6 +458,7 @@ def test_fused_append_in_the_grid_kernel_edge_positions(device, d, kv, ps):
 
 
 @pytest.mark.gpu
+@pytest.mark.routing("balanced")
 @pytest.mark.parametrize("hkv,group,D", [(8, 4, 128), (3, 2, 128), (16, 1, 128), (8, 4, 64), (2, 8, 64)])
 def test_balanced_schedule_records_the_parts_the_host_model_predicts(hkv, group, D):
     """The main kernel of the balanced schedule tells the merge kernel, per (sequence, KV head)
@@ -512,10 +513,11 @@ def test_balanced_schedule_records_the_parts_the_host_model_predicts(hkv, group,
 
 
 # ------------------------------------------------------------------ latency-bound calls: the library's own choice
+@pytest.mark.routing("balanced")
 @pytest.mark.parametrize("name,batch,ctx_hi,kv", [("llama3_8b_decode", 1, 500, None), ("llama3_8b_decode", 3, 2000, None),
                                                  ("llama32_1b_decode", 2, 300, None), ("llama32_1b_decode", 4, 1500, None),
                                                  ("llama3_70b_decode_fp8", 2, 1100, "fp8")])
-def test_small_calls_take_the_grid_schedule(device, monkeypatch, name, batch, ctx_hi, kv):
+def test_small_calls_take_the_grid_schedule(device, name, batch, ctx_hi, kv):
     """With partition_size = 0 a call over few short rows is routed to the grid schedule (whole rows
     when no row can exceed 640 tokens, 256-token partitions otherwise).  Same numbers as the balanced
     schedule to the tolerance between split sizes, same pools after the fused append, oracle parity,
@@ -524,11 +526,11 @@ def test_small_calls_take_the_grid_schedule(device, monkeypatch, name, batch, ct
     lib = _lib.load()
     w = workloads.make_workload("x", device=device, seed=11, shape=small(name, batch=batch, ctx_lo=40, ctx_hi=ctx_hi))
     k0, v0 = w.k_pool.clone(), w.v_pool.clone()
-    balanced = torch.full_like(w.query, float("nan"))           # the autouse fixture forces the balanced schedule
+    balanced = torch.full_like(w.query, float("nan"))           # routing "balanced": threshold 0
     ops.paged_decode_attn(balanced, w.query, w.k_pool, w.v_pool, w.block_table, w.context_lens, w.scale,
                           k_scale=w.k_scale, v_scale=w.v_scale, new_key=w.new_key, new_value=w.new_value)
     torch.cuda.synchronize()
-    monkeypatch.delenv("AICOMP_KV_SMALL_DECODE_TOKENS")
+    assert ops.set_small_decode_tokens(32768) == 0              # the library's default from here on
     s, mb = w.shape, w.block_table.shape[1]
     assert batch * mb * 16 <= 32768, "the case is meant to be below the default limit"
     qd, kd = ops._DT[w.query.dtype], ops._DT[w.k_pool.dtype]

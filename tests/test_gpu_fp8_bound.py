@@ -14,7 +14,8 @@ float32 source rows as the unquantised result:
     any row, n keys:
         |out_fp8 - out_unq| <= 1e-2 + min(0.3, 1.6 / sqrt(n))
 
-Measured on MI355X: decode at full size 8.4e-3 (sampled sequences, the shortest included);
+Measured on MI355X: decode at full size 8.4e-3 (sampled sequences, the shortest included; the
+test checks all 128);
 prefill rows 0.19 at 1-8 keys, 0.13 at 16, 0.09 at 32-64, 0.07 at 128, 0.06 at 256, 0.03 at 512,
 0.02 at 1024-2048 (six seeds, head_dim 64 and 128): between 1.6 and 3 times inside the rule.
 """
@@ -38,26 +39,26 @@ def fp8_atol_for_keys(n):
     return 1e-2 + np.minimum(0.3, 1.6 / np.sqrt(n))
 
 
+@pytest.mark.routing("balanced")            # a full-size batch: far above the routing threshold either way
 def test_fp8_decode_vs_unquantised_model_full_size(device):
     """Llama-3-70B per-GPU decode shape (batch 128, 64 / 8 heads, contexts 1024..8192) at full size:
-    fused append + decode over the fp8 pools, sampled sequences against float64 attention over the
-    float32 rows the pools were quantised from."""
+    fused append + decode over the fp8 pools, every one of the 128 sequences against float64
+    attention over the float32 rows the pools were quantised from."""
     w = workloads.make_workload("llama3_70b_decode_fp8", device=device)
     out = torch.full_like(w.query, float("nan"))
     ops.paged_decode_attn(out, w.query, w.k_pool, w.v_pool, w.block_table, w.context_lens, w.scale,
                           w.k_scale, w.v_scale, new_key=w.new_key, new_value=w.new_value)
     torch.cuda.synchronize()
-    order = sorted(range(w.num_seqs), key=lambda i: w.ctx_list[i])
-    sample = [order[0], order[len(order) // 2], order[-1], 5]
-    src = workloads.unquantised_context(w, sample)
     worst = 0.0
-    for s, (k, v) in zip(sample, src):
-        q = orc.decode_elements(raw(w.query[s:s + 1]), "bf16")
-        want = orc.attend_contiguous(q, k.double().cpu().numpy(), v.double().cpu().numpy(), w.scale)[0]
-        got = to_f64(out[s])
-        worst = max(worst, float(np.abs(got - want).max()))
-        assert_close_attn(got, want, FP8_ATOL, FP8_RTOL, f"fp8 decode vs unquantised, sequence {s}")
-    print(f"fp8 decode vs unquantised: max abs error {worst:.3e} over sequences {sample}")
+    for lo in range(0, w.num_seqs, 32):                       # 32 sequences' float32 source rows at a time
+        seqs = list(range(lo, min(lo + 32, w.num_seqs)))
+        for s, (k, v) in zip(seqs, workloads.unquantised_context(w, seqs)):
+            q = orc.decode_elements(raw(w.query[s:s + 1]), "bf16")
+            want = orc.attend_contiguous(q, k.double().cpu().numpy(), v.double().cpu().numpy(), w.scale)[0]
+            got = to_f64(out[s])
+            worst = max(worst, float(np.abs(got - want).max()))
+            assert_close_attn(got, want, FP8_ATOL, FP8_RTOL, f"fp8 decode vs unquantised, sequence {s}")
+    print(f"fp8 decode vs unquantised: max abs error {worst:.3e} over all {w.num_seqs} sequences")
 
 
 @pytest.mark.parametrize("d,hq,hkv", [(128, 16, 2), (64, 8, 2)])

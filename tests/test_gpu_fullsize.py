@@ -1,6 +1,7 @@
-"""The five benchmark shapes at their full sizes: properties that do not depend on the size
-(schedule agreement, fused == unfused, bit-exact scatter) plus the float64 oracle on a sample
-of sequences (the oracle walks tokens in Python, so a sample keeps the suite fast)."""
+"""The five benchmark shapes at their full sizes: the whole output tensor of every shape against
+the float64 oracle (every sequence, every prefill row; the oracle gathers each context with its
+vectorised gather, which tests/test_oracle.py pins against the token loop), plus properties that
+do not depend on the size (schedule agreement, fused == unfused, bit-exact scatter)."""
 import numpy as np
 import pytest
 import torch
@@ -13,14 +14,13 @@ pytestmark = pytest.mark.gpu
 BF16_ATOL, BF16_RTOL = 1e-2, 2e-2
 
 
-def oracle_rows(w, rows, q, bt, ctx):
+def oracle_decode_all(w, q, bt, ctx):
+    """Float64 oracle over every row of a decode batch (pools as they are on the device now)."""
     ks = None if w.k_scale is None else w.k_scale.cpu().numpy()
     vs = None if w.v_scale is None else w.v_scale.cpu().numpy()
-    kp, vp = raw(w.k_pool), raw(w.v_pool)
-    idx = torch.tensor(rows)
-    return orc.paged_decode_attn(raw(q[idx.to(q.device)]), kp, vp, bt.cpu().numpy()[rows],
-                                 [int(ctx[r]) for r in rows], w.scale, NAME[q.dtype], NAME[w.k_pool.dtype],
-                                 ks, vs)
+    return orc.paged_decode_attn(raw(q), raw(w.k_pool), raw(w.v_pool), bt.cpu().numpy(), [int(c) for c in ctx],
+                                 w.scale, NAME[q.dtype], NAME[w.k_pool.dtype], ks, vs,
+                                 gather=orc.gather_context_fast)
 
 
 def decode(w, q, bt, ctx, ps=0, **kw):
@@ -31,10 +31,10 @@ def decode(w, q, bt, ctx, ps=0, **kw):
     return out
 
 
-@pytest.mark.parametrize("name,sample", [("llama3_8b_decode", [0, 7, 31, 63]),
-                                         ("long_context_skewed", None),
-                                         ("llama3_70b_decode_fp8", [0, 64, 127])])
-def test_full_decode_shapes(device, name, sample):
+@pytest.mark.parametrize("name", ["llama3_8b_decode", "long_context_skewed", "llama3_70b_decode_fp8"])
+def test_full_decode_shapes(device, name):
+    """Configs 2, 3 and 5: every sequence of the batch within 1e-2 abs or 2e-2 rel of the float64
+    oracle (for the fp8 pools: the oracle over the dequantised codes)."""
     w = workloads.make_workload(name, device=device)
     k0, v0 = w.k_pool.clone(), w.v_pool.clone()
     # fused append + decode (balanced schedule) on a copy of the pools
@@ -50,12 +50,9 @@ def test_full_decode_shapes(device, name, sample):
     grid = decode(w, w.query, w.block_table, w.context_lens, ps=1024)
     assert (grid.float() - balanced.float()).abs().max() <= 2e-3
     assert torch.isfinite(balanced.float()).all()
-    if sample is None:                                          # the two longest and the shortest
-        order = sorted(range(w.num_seqs), key=lambda i: w.ctx_list[i])
-        sample = [order[0], order[-2], order[-1]]
-    want = oracle_rows(w, sample, w.query, w.block_table, w.ctx_list)
-    got = to_f64(balanced)[sample]
-    assert_close_attn(got, want, BF16_ATOL, BF16_RTOL, f"{name} rows {sample}")
+    want = oracle_decode_all(w, w.query, w.block_table, w.ctx_list)
+    assert_close_attn(to_f64(balanced), want, BF16_ATOL, BF16_RTOL, f"{name}, all {w.num_seqs} sequences")
+    assert_close_attn(to_f64(grid), want, BF16_ATOL, BF16_RTOL, f"{name}, grid schedule, all sequences")
 
 
 def test_full_long_context_unsplit_equals_split(device):
@@ -93,10 +90,13 @@ def test_full_chunked_prefill_mixed(device):
     qd = w.query[last].contiguous()
     d2 = decode(w, qd, w.block_table[:npre].contiguous(), w.context_lens[:npre].contiguous())
     assert (d2.float() - out[last].float()).abs().max() <= 4e-3
-    want = oracle_rows(w, [npre, npre + 59], w.query[T - npre:], w.block_table, w.ctx_list)
-    # (rows npre.. of the decode part: index into the decode queries)
-    got = to_f64(dec)[[0, 59]]
-    assert_close_attn(got, want, BF16_ATOL, BF16_RTOL, "decode tail of the mixed step")
+    # config 4, whole output: all 2048 prefill rows and all 60 decode rows against the float64 oracle
+    want = orc.paged_prefill_attn(raw(w.query[:T]), raw(w.k_pool), raw(w.v_pool), w.block_table.cpu().numpy()[:npre],
+                                  w.ctx_list[:npre], w.cu_q_lens.cpu().numpy()[:npre + 1], w.scale, "bf16", "bf16",
+                                  gather=orc.gather_context_fast)
+    assert_close_attn(to_f64(out), want, BF16_ATOL, BF16_RTOL, "all prefill rows of the mixed step")
+    want = oracle_decode_all(w, w.query[T:], w.block_table[npre:], w.ctx_list[npre:])
+    assert_close_attn(to_f64(dec), want, BF16_ATOL, BF16_RTOL, "all decode rows of the mixed step")
 
 
 def test_full_fp32_anchor_vs_cpu_reference_path(device):

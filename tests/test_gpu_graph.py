@@ -93,14 +93,13 @@ def test_fused_decode_step_replays_under_a_graph(device, kv_dtype):
 
 
 @pytest.mark.parametrize("B,d,prompt", [(2, 64, 37), (4, 128, 600)])
-def test_adapter_decode_step_replays_from_a_graph(device, monkeypatch, B, d, prompt):
+def test_adapter_decode_step_replays_from_a_graph(device, B, d, prompt):
     """Two layers of the drop-in operator with device-side positions: one decode step (both layers)
     is captured once and replayed with new inputs; every replay equals the same step made eagerly by
-    a twin pair of operators, bit for bit, and the host positions agree after ``advance``.  Runs with
-    the library's own schedule choice (these sizes take the grid schedule) and eager work between
-    the replays."""
+    a twin pair of operators, bit for bit, and the host positions agree after ``advance``.  Runs under
+    both routings (with the library's own choice these sizes take the grid schedule) and with eager
+    work between the replays."""
     from aicomp_amd import kv_cache as akv
-    monkeypatch.delenv("AICOMP_KV_SMALL_DECODE_TOKENS")
     hq, g = 8, 4
     hkv = hq // g
     gen = torch.Generator().manual_seed(3)

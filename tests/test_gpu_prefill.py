@@ -190,22 +190,11 @@ def test_config4_chunked_prefill_reduced(device):
                            w.block_table[:npre].contiguous(), w.context_lens[:npre].contiguous(),
                            w.cu_q_lens[:npre + 1].contiguous(), w.scale, max_q_len=512)
     torch.cuda.synchronize()
-    # oracle on a sample of rows of every chunk (first, last, tile boundaries, random)
-    rng = np.random.default_rng(0)
-    kp, vp, tab = raw(w.k_pool), raw(w.v_pool), w.block_table.cpu().numpy()
-    qraw = raw(w.query)
-    got = to_f64(out)
-    for sidx in range(npre):
-        n, L = w.new_list[sidx], w.ctx_list[sidx]
-        prior = L - n
-        rows = sorted(set([0, 1, 15, 16, 63, 64, 255, 511] + rng.integers(0, n, 6).tolist()))
-        k = orc.decode_elements(orc.gather_context(kp, tab[sidx], L), "bf16")
-        v = orc.decode_elements(orc.gather_context(vp, tab[sidx], L), "bf16")
-        for i in rows:
-            r = int(w.cu_q_lens[sidx]) + i
-            qv = orc.decode_elements(qraw[r], "bf16")[None]
-            want = orc.attend_contiguous(qv, k[: prior + i + 1], v[: prior + i + 1], w.scale)[0]
-            assert_close_attn(got[r], want, BF16_ATOL, BF16_RTOL, f"chunk {sidx} row {i}")
+    # every row of every chunk against the float64 oracle
+    want = orc.paged_prefill_attn(raw(w.query[:T]), raw(w.k_pool), raw(w.v_pool), w.block_table.cpu().numpy()[:npre],
+                                  w.ctx_list[:npre], w.cu_q_lens.cpu().numpy()[:npre + 1], w.scale, "bf16", "bf16",
+                                  gather=orc.gather_context_fast)
+    assert_close_attn(to_f64(out), want, BF16_ATOL, BF16_RTOL, "all rows of the four chunks")
 
 
 # ------------------------------------------------------------------ head_dim 64 on the matrix-core kernel
@@ -253,11 +242,11 @@ def test_prefill_context_shorter_than_chunk_gives_zero_rows(device, dtype):
     assert_close_attn(to_f64(got)[keep], want[keep], tol[0], tol[1], "chunks beside the inconsistent one")
 
 
-def test_long_prompt_sampled_rows_and_scaling_in_v(device):
+def test_long_prompt_all_rows_and_scaling_in_v(device):
     """One fresh prompt of 4096 tokens at the Llama-3-8B head shape (the size class of the long-prompt
-    bench shapes).  The float64 oracle is run on sampled rows only (a full pass takes minutes on the
-    CPU); on all rows the size-independent property is checked that doubling V doubles the output bit
-    for bit (the probabilities do not depend on V, and a factor of two is exact in bf16)."""
+    bench shapes): every row against the float64 oracle, and the size-independent property that
+    doubling V doubles the output bit for bit (the probabilities do not depend on V, and a factor of
+    two is exact in bf16)."""
     n = 4096
     c = build_case(device, priors=[0], news=[n], hq=32, hkv=8, d=128, seed=31, poison=True)
     got = run(c)
@@ -265,14 +254,8 @@ def test_long_prompt_sampled_rows_and_scaling_in_v(device):
     c2 = dict(c, v_pool=(c["v_pool"].float() * 2).to(torch.bfloat16))
     got2 = run(c2)
     assert torch.equal((got.float() * 2).to(torch.bfloat16).view(torch.int16), got2.view(torch.int16))
-    rng = np.random.default_rng(5)
     kp = torch.nan_to_num(c["k_pool"].float().cpu(), nan=0.0, posinf=0.0).to(torch.bfloat16)
     vp = torch.nan_to_num(c["v_pool"].float().cpu(), nan=0.0, posinf=0.0).to(torch.bfloat16)
-    tab = c["table"].cpu().numpy()
-    k = orc.decode_elements(orc.gather_context(raw(kp), tab[0], n), "bf16")
-    v = orc.decode_elements(orc.gather_context(raw(vp), tab[0], n), "bf16")
-    qraw, g64 = raw(c["q"]), to_f64(got)
-    for i in sorted(set([0, 1, 63, 64, 127, 128, 2047, 2048, n - 65, n - 64, n - 1] + rng.integers(0, n, 8).tolist())):
-        qv = orc.decode_elements(qraw[i], "bf16")[None]
-        want = orc.attend_contiguous(qv, k[: i + 1], v[: i + 1], c["scale"])[0]
-        assert_close_attn(g64[i], want, BF16_ATOL, BF16_RTOL, f"row {i}")
+    want = orc.paged_prefill_attn(raw(c["q"]), raw(kp), raw(vp), c["table"].cpu().numpy(), [n], [0, n], c["scale"],
+                                  "bf16", "bf16", gather=orc.gather_context_fast)
+    assert_close_attn(to_f64(got), want, BF16_ATOL, BF16_RTOL, "4096-token prompt, all rows")

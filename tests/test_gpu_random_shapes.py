@@ -27,11 +27,11 @@ def _close(got, want, atol, rtol):
 
 @pytest.mark.parametrize("seed", range(4))
 @pytest.mark.parametrize("schedule", ["balanced", "library"])
-def test_random_decode_and_prefill_shapes(device, monkeypatch, seed, schedule):
+def test_random_decode_and_prefill_shapes(device, seed, schedule):
     # "library": the library's own choice of decode schedule for small calls (the suite otherwise
     # pins automatic calls to the balanced schedule)
     if schedule == "library":
-        monkeypatch.delenv("AICOMP_KV_SMALL_DECODE_TOKENS")
+        ops.set_small_decode_tokens(32768)          # the autouse fixture restores the suite's setting
     rnd = random.Random(100 + seed)
     for trial in range(12):
         nseq = rnd.randint(1, 5)
@@ -67,9 +67,9 @@ def test_random_decode_and_prefill_shapes(device, monkeypatch, seed, schedule):
 
 @pytest.mark.parametrize("seed", range(3))
 @pytest.mark.parametrize("schedule", ["balanced", "library"])
-def test_random_operator_sessions(device, monkeypatch, seed, schedule):
+def test_random_operator_sessions(device, seed, schedule):
     if schedule == "library":
-        monkeypatch.delenv("AICOMP_KV_SMALL_DECODE_TOKENS")
+        ops.set_small_decode_tokens(32768)          # the autouse fixture restores the suite's setting
     rnd = random.Random(200 + seed)
     torch.manual_seed(200 + seed)
     for trial in range(10):

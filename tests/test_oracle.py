@@ -123,12 +123,36 @@ def test_append_gather_round_trip_and_sentinels():
     for s, L in enumerate(lens):
         assert np.array_equal(orc.gather_context(k_pool, table[s], L), key[cur:cur + L])
         assert np.array_equal(orc.gather_context(v_pool, table[s], L), val[cur:cur + L])
+        # the vectorised gather the full-size tests use is the token loop, element for element
+        assert np.array_equal(orc.gather_context_fast(k_pool, table[s], L), key[cur:cur + L])
+        assert orc.gather_context_fast(v_pool, table[s], L).shape == (L, hkv, d)
         cur += L
     touched = np.zeros(nb * bs, dtype=bool)
     touched[slots] = True
     flat_k = k_pool.transpose(0, 2, 1, 3).reshape(nb * bs, hkv, d)
     assert (flat_k[~touched] == 0xBEEF).all()
     assert len(set(slots)) == len(slots)
+
+
+def test_vectorised_gather_equals_the_token_loop_in_the_attention_oracle():
+    """paged_decode_attn / paged_prefill_attn give identical float64 results with either gather,
+    on ragged lengths that end inside a block, at a block edge and on an empty row."""
+    rng = np.random.default_rng(7)
+    hq, hkv, d, bs, nb = 4, 2, 8, 4, 64
+    lens = [1, 4, 5, 17, 0, 33]
+    table = _rand_table(rng, [max(L, 1) for L in lens], bs, nb)
+    kp = rng.standard_normal((nb, hkv, bs, d)).astype(np.float32)
+    vp = rng.standard_normal((nb, hkv, bs, d)).astype(np.float32)
+    q = rng.standard_normal((len(lens), hq, d)).astype(np.float32)
+    a = orc.paged_decode_attn(q, kp, vp, table, lens, 0.3)
+    b = orc.paged_decode_attn(q, kp, vp, table, lens, 0.3, gather=orc.gather_context_fast)
+    assert np.array_equal(a, b)
+    news = [1, 2, 5, 9, 0, 20]
+    cu = np.concatenate([[0], np.cumsum(news)])
+    qq = rng.standard_normal((cu[-1], hq, d)).astype(np.float32)
+    a = orc.paged_prefill_attn(qq, kp, vp, table, lens, cu, 0.3)
+    b = orc.paged_prefill_attn(qq, kp, vp, table, lens, cu, 0.3, gather=orc.gather_context_fast)
+    assert np.array_equal(a, b)
 
 
 def test_append_equals_reference_slice_assign():
