@@ -29,7 +29,7 @@ SYMBOLS = (
 
 F32, BF16, FP8_E4M3, F16 = 0, 1, 2, 3
 
-_lock = threading.Lock()
+_lock = threading.RLock()       # torch_ops() loads the HIP library while holding it
 _lib = None
 
 
@@ -90,6 +90,28 @@ def load() -> C.CDLL:
             _declare(lib)
             _lib = lib
         return _lib
+
+
+TORCH_LIB_PATH = os.path.join(_HERE, "libaicomp_kv_torch.so")
+_torch_ns = None
+
+
+def torch_ops():
+    """The ``torch.ops.mi355_kv`` namespace (``kv_append``, ``paged_decode_attn``,
+    ``paged_decode_attn_append``, ``paged_prefill_attn``, ``decode_step``): the C ABI registered as
+    PyTorch operators by csrc/torch_ops.cpp, built by ``python -m aicomp_amd.build``.  Loads the
+    registration library on first use; raises ``LibraryMissing`` if it was not built."""
+    global _torch_ns
+    if _torch_ns is None:
+        with _lock:
+            if _torch_ns is None:
+                if not os.path.exists(TORCH_LIB_PATH):
+                    raise LibraryMissing(f"{TORCH_LIB_PATH} is missing: build it with `python -m aicomp_amd.build`")
+                import torch
+                load()                              # the HIP library it links against, checked first
+                torch.ops.load_library(TORCH_LIB_PATH)
+                _torch_ns = torch.ops.mi355_kv
+    return _torch_ns
 
 
 def check(rc: int, lib: C.CDLL) -> None:

@@ -49,6 +49,29 @@ def build(verbose: bool = True, jobs: int = 8) -> str:
     return LIB
 
 
+TORCH_LIB = os.path.join(HERE, "libaicomp_kv_torch.so")
+
+
+def build_torch_ops(verbose: bool = True) -> str:
+    """Compile csrc/torch_ops.cpp: the TORCH_LIBRARY(mi355_kv) registration of the C ABI (host code
+    only: it links libaicomp_kv.so and libtorch, and holds no device code)."""
+    import torch
+    from torch.utils import cpp_extension as ce
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    abi = int(torch.compiled_with_cxx11_abi())
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1",
+           "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={abi}", *[f"-I{d}" for d in ce.include_paths()],
+           "-I/opt/rocm/include", os.path.join(CSRC, "torch_ops.cpp"), "-o", TORCH_LIB, f"-L{tlib}", "-ltorch",
+           "-ltorch_cpu", "-lc10", "-ltorch_hip", "-lc10_hip", f"-L{HERE}", "-laicomp_kv", "-Wl,-rpath,$ORIGIN",
+           f"-Wl,-rpath,{tlib}"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"compiling torch_ops.cpp failed:\n{r.stdout}\n{r.stderr}")
+    if verbose:
+        print(f"built {TORCH_LIB}")
+    return TORCH_LIB
+
+
 def build_host_example(verbose: bool = True) -> str:
     """Compile tests/cabi_host.cpp, a C++ program that links the library directly (no Python, no
     torch): the boundary as a C or C++ host sees it."""
@@ -67,5 +90,6 @@ def build_host_example(verbose: bool = True) -> str:
 
 if __name__ == "__main__":
     build()
+    build_torch_ops()
     build_host_example()
     sys.exit(0)

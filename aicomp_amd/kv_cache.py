@@ -40,10 +40,19 @@ from typing import Dict, Optional, Tuple
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
+import torch.nn.modules.module as _nn_module
 
-from . import ops
+from . import _lib, ops
 
 BLOCK_SIZE = 16
+
+# The decode step as one registered PyTorch operator (a third of the host time of the ctypes
+# route at batch 1).  Both routes end in the same C entry point of the HIP library; the ctypes
+# one remains for device-side positions and for installations without the registration library.
+try:
+    _TORCH_DECODE = _lib.torch_ops().decode_step.default
+except _lib.LibraryMissing:
+    _TORCH_DECODE = None
 
 
 def _detect_group(key: torch.Tensor) -> int:
@@ -77,6 +86,7 @@ class _PagedLayer:
     def __init__(self, batch: int, kv_heads: int, head_dim: int, max_seq_len: int,
                  dtype: torch.dtype, device: torch.device, block_size: int = BLOCK_SIZE):
         self.batch, self.kv_heads, self.head_dim = batch, kv_heads, head_dim
+        self.default_scale = 1.0 / math.sqrt(head_dim)
         self.max_seq_len, self.block_size = max_seq_len, block_size
         self.blocks_per_seq = max(1, math.ceil(max_seq_len / block_size))
         nb = batch * self.blocks_per_seq
@@ -122,6 +132,11 @@ class _PagedLayer:
         key/value ``[B, H, 1, D]`` written at position pos.  With ``live`` the position is the
         device-side counter ``live_ctx`` (advanced here by a one-element-per-sequence kernel), so
         the step can be captured into a HIP graph and replayed."""
+        if not live and _TORCH_DECODE is not None:
+            # one dispatch through torch.ops.mi355_kv.decode_step: checks, output allocation,
+            # current stream and the fused append + decode call all happen in C++
+            return _TORCH_DECODE(query, key, value, self.k_pool, self.v_pool, self.block_table, self.ctx_rows, pos,
+                                 group, scale, None)
         Hq = query.shape[1]
         call = self._decode.get((Hq, query.dtype, scale))
         if call is None:
@@ -133,12 +148,13 @@ class _PagedLayer:
         if live:
             # the counter moves only once the call's arguments have passed their checks (a rejected
             # call must leave it where it was); add_ is a fill-type kernel, safe inside a captured graph
-            ctx, ready = self.live_ctx.data_ptr(), self._bump_live
+            ctx, ready, width = self.live_ctx.data_ptr(), self._bump_live, None
         else:
-            # row pos + 1 of the context-length table, by address (a view tensor costs microseconds)
-            ctx, ready = self._ctx_base + (pos + 1) * self._ctx_pitch, None
+            # row pos + 1 of the context-length table, by address (a view tensor costs microseconds);
+            # only the table columns that hold those pos + 1 tokens are in use
+            ctx, ready, width = self._ctx_base + (pos + 1) * self._ctx_pitch, None, pos // self.block_size + 1
         # [B, Hq, 1, D] has the memory layout of [B, Hq, D]: the call takes the tensors as they are
-        return call.step4d(torch.empty_like(query), query, key, value, group, ctx, ready)
+        return call.step4d(torch.empty_like(query), query, key, value, group, ctx, ready, width)
 
     def _bump_live(self) -> None:
         self.live_ctx.add_(1)
@@ -488,9 +504,31 @@ class CachedScaledDotProductAttention(nn.Module):
         self.cache_pos = 0
         self._device_positions = False          # the next use_device_positions() starts the counter afresh
 
+    def __call__(self, *args, **kwargs):
+        # One call per layer and token at batch 1 is bound by the host: nn.Module's hook dispatch
+        # costs a microsecond per call and is only taken when some hook is actually registered.
+        if (self._forward_hooks or self._forward_pre_hooks or self._backward_hooks or self._backward_pre_hooks
+                or _nn_module._global_forward_hooks or _nn_module._global_forward_pre_hooks
+                or _nn_module._global_backward_hooks or _nn_module._global_backward_pre_hooks):
+            return super().__call__(*args, **kwargs)
+        return self.forward(*args, **kwargs)
+
     def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                 attn_mask: Optional[torch.Tensor] = None, dropout_p: float = 0.0,
                 is_causal: bool = False, **kwargs) -> torch.Tensor:
+        # decode step on the operator's own cache, the call a generation loop makes once per layer
+        # and token: straight to the registered operator (checks, output, stream and launch in C++)
+        store = self._store
+        if (store is not None and self._enabled and self.kv_manager is None and not self._device_positions
+                and _TORCH_DECODE is not None and dropout_p == 0.0 and query.dim() == 4 and query.shape[2] == 1
+                and key.dtype == store.k_pool.dtype):
+            pos = self.cache_pos
+            if pos < self.max_seq_len:
+                scale = kwargs.get("scale")
+                out = _TORCH_DECODE(query, key, value, store.k_pool, store.v_pool, store.block_table, store.ctx_rows,
+                                    pos, self._group, store.default_scale if scale is None else float(scale), None)
+                self.cache_pos = pos + 1
+                return out
         if not self._enabled:
             return F.scaled_dot_product_attention(query, key, value, attn_mask=attn_mask,
                                                   dropout_p=dropout_p, is_causal=is_causal, **kwargs)

@@ -293,14 +293,16 @@ class PreparedDecode:
         return out
 
     def step4d(self, out: torch.Tensor, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
-               group: int, context_lens, ready=None) -> torch.Tensor:
+               group: int, context_lens, ready=None, width: Optional[int] = None) -> torch.Tensor:
         """The fused append + decode call on the operator's own tensors: ``query`` / ``out``
         ``[B, Hq, 1, D]`` contiguous, ``key`` / ``value`` ``[B, H, 1, D]`` with H = Hkv or
         Hkv * group (heads repeated ``group`` times, as HF's ``repeat_kv`` leaves them: every
         group-th head is read).  No view tensors are made: the strides go to the library as they
         are.  ``context_lens`` is an int32 ``[B]`` tensor on the device, or its device address.
         ``ready``, if given, is called once the arguments have passed every check, right before
-        the launch (for work that must not happen for a rejected call)."""
+        the launch (for work that must not happen for a rejected call).  ``width`` (at most the
+        table's width) tells the library how many table columns are in use, so that it sizes the
+        split for the contexts as they are now."""
         B, Hq, D = self.q_shape
         hkv = self.kv_shape[1]
         H = key.shape[1]
@@ -319,10 +321,13 @@ class PreparedDecode:
         ws_ptr, ws_bytes = (None, 0) if ws is None else (ws.data_ptr(), ws.numel())
         if ready is not None:
             ready()
+        tail = self._tail
+        if width is not None and 0 < width < tail[5]:
+            tail = tail[:5] + (width,) + tail[6:]
         rc = self.lib.aicomp_paged_decode_attn_append(
             out.data_ptr(), query.data_ptr(), key.data_ptr(), value.data_ptr(),
             key.stride(0), key.stride(1) * hstep, *self._head,
-            context_lens if isinstance(context_lens, int) else context_lens.data_ptr(), *self._tail,
+            context_lens if isinstance(context_lens, int) else context_lens.data_ptr(), *tail,
             ws_ptr, ws_bytes, stream)
         _lib.check(rc, self.lib)
         return out

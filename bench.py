@@ -367,6 +367,51 @@ def small_batch_decode_bench(dev):
     return {"shape": "32 query / 8 KV heads, head_dim 64, bf16", "calls": out_rows}
 
 
+def host_cost_bench(dev):
+    """Host time of ONE decode call of the drop-in operator at the size the reference's own engine
+    runs (batch 1, Llama-3.2-1B heads: 32 / 8, head_dim 64, bf16, K/V arriving expanded by
+    repeat_kv): the Python thread's time per call, timed over 1000 calls without a synchronisation
+    inside (the position is set back before every call, so each call sees the stated context).
+    At 600 cached tokens the call is one launch (whole rows), at 1500 two (256-token partitions and
+    their merge).  Through the registered operator (torch.ops.mi355_kv.decode_step) and through the
+    ctypes binding of the same C entry point."""
+    import torch
+    from aicomp_amd import kv_cache as akv
+    B, hq, g, d = 1, 32, 4, 64
+    hkv = hq // g
+    mk = lambda n, h: torch.randn(B, h, n, d, device=dev).to(torch.bfloat16)
+    res = {"shape": "batch 1, 32 query / 8 KV heads (K/V expanded to 32), head_dim 64, bf16"}
+    for name, route in (("torch_op", akv._TORCH_DECODE), ("ctypes", None)):
+        if name == "torch_op" and route is None:
+            continue
+        saved, akv._TORCH_DECODE = akv._TORCH_DECODE, route
+        try:
+            op = akv.CachedScaledDotProductAttention(0, 2048, num_kv_groups=g)
+            op.enable()
+            op(mk(1500, hq), mk(1500, hkv).repeat_interleave(g, 1), mk(1500, hkv).repeat_interleave(g, 1), is_causal=True)
+            q, k, v = mk(1, hq), mk(1, hkv).repeat_interleave(g, 1), mk(1, hkv).repeat_interleave(g, 1)
+            for ctx in (600, 1500):
+                for _ in range(200):
+                    op.cache_pos = ctx
+                    op(q, k, v)
+                torch.cuda.synchronize()
+                best = None
+                for _ in range(5):
+                    n = 1000
+                    t0 = time.perf_counter()
+                    for _ in range(n):
+                        op.cache_pos = ctx
+                        op(q, k, v)
+                    host = (time.perf_counter() - t0) / n
+                    torch.cuda.synchronize()
+                    best = host if best is None else min(best, host)
+                res[f"host_us_per_call_{name}_ctx{ctx}"] = round(best * 1e6, 2)
+        finally:
+            akv._TORCH_DECODE = saved
+    res["host_us_per_call"] = res.get("host_us_per_call_torch_op_ctx600", res.get("host_us_per_call_ctypes_ctx600"))
+    return res
+
+
 def sampler_bench(dev, batch=64, vocab=128256, temperature=0.8, top_k=50, top_p=0.9, reps=20):
     """The step after the attention path: one token per row of [64, 128256] fp32 logits with
     temperature / top-k / top-p (opt_prime/opt_prime/inference.py:786-843).  Beside the kernel, the
@@ -750,6 +795,7 @@ def main():
         "step_planner": planner_bench(dev),
         "sampler": sampler_bench(dev),
         "decode_small_batch": small_batch_decode_bench(dev),
+        "operator_host_cost": host_cost_bench(dev),
         "prefill_other_shapes": prefill_shapes_bench(dev),
     }
     if not args.no_cpu:

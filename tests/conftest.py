@@ -57,3 +57,15 @@ def decode_routing(request):
         return
     yield mode
     ops.set_small_decode_tokens(prev)
+
+
+@pytest.fixture(params=["torch_op", "ctypes"])
+def host_route(request, monkeypatch):
+    """The two host routes of the drop-in operator's decode step into the HIP library: the
+    registered PyTorch operator (torch.ops.mi355_kv.decode_step) and the ctypes binding."""
+    from aicomp_amd import kv_cache as akv
+    if request.param == "ctypes":
+        monkeypatch.setattr(akv, "_TORCH_DECODE", None)
+    else:
+        assert akv._TORCH_DECODE is not None, "libaicomp_kv_torch.so is not built"
+    return request.param

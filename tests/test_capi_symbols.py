@@ -93,3 +93,16 @@ def test_routing_threshold_is_one_word_shared_by_sizing_and_calls():
         assert ops.set_small_decode_tokens(0) == 0 and ops._route_epoch == e0 + 1
     finally:
         lib.aicomp_kv_set_small_decode_tokens(prev)
+
+
+def test_torch_operator_library_registers_the_named_ops():
+    """libaicomp_kv_torch.so (built from csrc/torch_ops.cpp) registers the C ABI under
+    torch.ops.mi355_kv with the signatures the integration notes give; loading needs no GPU."""
+    ns = _lib.torch_ops()
+    for name in ("kv_append", "paged_decode_attn", "paged_decode_attn_append", "paged_prefill_attn", "decode_step"):
+        assert hasattr(ns, name), name
+    s = str(ns.paged_decode_attn.default._schema)
+    assert s.startswith("mi355_kv::paged_decode_attn(Tensor(a!) out, Tensor query, Tensor k_pool, Tensor v_pool, "
+                        "Tensor block_table, Tensor context_lens, float scale")
+    assert "Tensor(a!) k_pool" in str(ns.kv_append.default._schema)
+    assert str(ns.decode_step.default._schema).endswith("-> Tensor")

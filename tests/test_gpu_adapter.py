@@ -39,7 +39,7 @@ def _run_session(op_new, op_ref, B, hq, g, d, steps, device, dtype, atol):
         assert op_new.cache_pos == op_ref.pos
 
 
-def test_adapter_llama_shape_bf16_internal(device):
+def test_adapter_llama_shape_bf16_internal(device, host_route):
     """Llama-3-8B head geometry, batch 3: prefill 300 then 6 decode steps, K/V arriving expanded
     to 32 heads the way HF Llama passes them; the reference semantics run in fp32 on the same
     bf16-rounded inputs."""
@@ -58,7 +58,7 @@ def test_adapter_llama_shape_bf16_internal(device):
     assert new.cache_k is None and not new._enabled
 
 
-def test_adapter_external_manager_bf16(device):
+def test_adapter_external_manager_bf16(device, host_route):
     B, hq, g, d = 2, 16, 4, 128
     mgr = akv.KVCacheManager(num_layers=2, max_batch_size=4, max_seq_len=256, num_heads=hq, head_dim=d,
                              dtype=torch.bfloat16, device=device, num_kv_heads=hq // g)
@@ -105,7 +105,7 @@ def test_adapter_chunked_prefill_is_causal(device):
     assert a.cache_pos == b.cache_pos == 29
 
 
-def test_adapter_llama32_1b_heads_bf16(device):
+def test_adapter_llama32_1b_heads_bf16(device, host_route):
     """The model of the reference's examples (Llama-3.2-1B: 32 query / 8 KV heads of 64): prefill of an
     odd length, decode steps across a block boundary, K/V arriving expanded by repeat_kv."""
     B, hq, g, d = 2, 32, 4, 64
@@ -117,7 +117,7 @@ def test_adapter_llama32_1b_heads_bf16(device):
     new.disable()
 
 
-def test_adapter_batch_one_and_hf_style_views(device):
+def test_adapter_batch_one_and_hf_style_views(device, host_route):
     """Batch 1 (what the reference's examples run) with q/k/v arriving the way HF Llama builds them:
     ``proj(x).view(B, n, H, D).transpose(1, 2)``, i.e. non-contiguous views; for batch 1 the
     token-major reshape of such a tensor is itself a strided view."""
@@ -151,11 +151,19 @@ def test_adapter_batch_one_and_hf_style_views(device):
     new.disable()
 
 
-def test_manager_mode_decode_is_one_fused_call_and_equals_internal_mode(device):
+@pytest.mark.parametrize("route", ["torch_op", "ctypes"])
+def test_manager_mode_decode_is_one_fused_call_and_equals_internal_mode(device, monkeypatch, route):
     """With a manager attached (the engine's ``--use-kv-manager`` mode, kv_cache.py:378-381) a decode
     step takes the same fused append + attention call as internal mode: one library call per layer
-    and token, output and pools bit-identical to the internal-mode operator."""
+    and token, output and pools bit-identical to the internal-mode operator.  Both host routes to
+    the library: the registered PyTorch operator and the ctypes binding."""
     from aicomp_amd import _lib
+    if route == "ctypes":
+        monkeypatch.setattr(akv, "_TORCH_DECODE", None)
+    else:
+        real_op = akv._TORCH_DECODE
+        assert real_op is not None
+        monkeypatch.setattr(akv, "_TORCH_DECODE", lambda *a: (calls.append("torch_op.decode_step"), real_op(*a))[1])
     B, hq, g, d, layers = 3, 16, 4, 128, 2
     hkv = hq // g
     mgr = akv.KVCacheManager(num_layers=layers, max_batch_size=4, max_seq_len=128, num_heads=hq, head_dim=d,
@@ -172,6 +180,7 @@ def test_manager_mode_decode_is_one_fused_call_and_equals_internal_mode(device):
     calls = []
     # every entry point that launches work (the sizing helpers are host arithmetic)
     names = [s for s in _lib.SYMBOLS if s not in ("aicomp_kv_version", "aicomp_kv_last_error",
+                                                  "aicomp_kv_set_small_decode_tokens",
                                                   "aicomp_paged_decode_workspace_bytes",
                                                   "aicomp_paged_decode_partition_size")]
     real = {s: getattr(lib, s) for s in names}
@@ -196,7 +205,7 @@ def test_manager_mode_decode_is_one_fused_call_and_equals_internal_mode(device):
                     setattr(lib, s, real[s])
             assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"n={n} layer {layer}"
             if n == 1:
-                assert calls == ["aicomp_paged_decode_attn_append"], calls
+                assert calls == (["aicomp_paged_decode_attn_append"] if route == "ctypes" else ["torch_op.decode_step"]), calls
             else:
                 assert calls == ["aicomp_kv_append", "aicomp_paged_prefill_attn"], calls
         assert mgr.get_seq_len() == ext[0].cache_pos == own[0].cache_pos

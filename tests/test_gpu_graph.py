@@ -93,13 +93,22 @@ def test_fused_decode_step_replays_under_a_graph(device, kv_dtype):
 
 
 @pytest.mark.parametrize("B,d,prompt", [(2, 64, 37), (4, 128, 600)])
-def test_adapter_decode_step_replays_from_a_graph(device, B, d, prompt):
+def test_adapter_decode_step_replays_from_a_graph(device, decode_routing, B, d, prompt):
     """Two layers of the drop-in operator with device-side positions: one decode step (both layers)
     is captured once and replayed with new inputs; every replay equals the same step made eagerly by
     a twin pair of operators, bit for bit, and the host positions agree after ``advance``.  Runs under
     both routings (with the library's own choice these sizes take the grid schedule) and with eager
     work between the replays."""
     from aicomp_amd import kv_cache as akv
+    # A replayed step cannot know its position on the host, so it sizes the split for the whole
+    # table; the eager twin sizes it for the context as it is.  On the balanced schedule the tiles
+    # are dealt the same way either way (bit-identical results); under the library's own routing
+    # the two may take different splits, which agree to the tolerance between split sizes.
+    def same(a, b, what=""):
+        if decode_routing == "balanced":
+            assert torch.equal(a.view(torch.int16), b.view(torch.int16)), what
+        else:
+            assert (a.float() - b.float()).abs().max().item() <= 2e-3, what
     hq, g = 8, 4
     hkv = hq // g
     gen = torch.Generator().manual_seed(3)
@@ -145,7 +154,7 @@ def test_adapter_decode_step_replays_from_a_graph(device, B, d, prompt):
         assert [op.cache_pos for op in graph_ops] == pos_before, "a recorded call is not a step"
     torch.cuda.synchronize()
     for i in range(2):
-        assert torch.equal(got0[i].view(torch.int16), want[0][i].view(torch.int16))
+        same(got0[i], want[0][i])
     filler = torch.empty(1 << 24, dtype=torch.uint8, device=device)
     for t in range(1, steps):
         for i in range(2):
@@ -155,7 +164,7 @@ def test_adapter_decode_step_replays_from_a_graph(device, B, d, prompt):
         graph.replay()
         torch.cuda.synchronize()
         for i in range(2):
-            assert torch.equal(out_s[i].view(torch.int16), want[t][i].view(torch.int16)), f"replay {t}, layer {i}"
+            same(out_s[i], want[t][i], f"replay {t}, layer {i}")
     for op in graph_ops:
         op.advance(steps - 1)
     assert [op.cache_pos for op in graph_ops] == [op.cache_pos for op in eager_ops] == [prompt + steps] * 2
@@ -163,4 +172,4 @@ def test_adapter_decode_step_replays_from_a_graph(device, B, d, prompt):
     for i in range(2):
         assert torch.equal(graph_ops[i].cache_k.view(torch.int16), eager_ops[i].cache_k.view(torch.int16))
         q, k, v = mk(1, hq), expand(mk(1, hkv)), expand(mk(1, hkv))
-        assert torch.equal(graph_ops[i](q, k, v).view(torch.int16), eager_ops[i](q, k, v).view(torch.int16))
+        same(graph_ops[i](q, k, v), eager_ops[i](q, k, v))

@@ -67,7 +67,7 @@ def test_random_decode_and_prefill_shapes(device, seed, schedule):
 
 @pytest.mark.parametrize("seed", range(3))
 @pytest.mark.parametrize("schedule", ["balanced", "library"])
-def test_random_operator_sessions(device, seed, schedule):
+def test_random_operator_sessions(device, seed, schedule, host_route):
     if schedule == "library":
         ops.set_small_decode_tokens(32768)          # the autouse fixture restores the suite's setting
     rnd = random.Random(200 + seed)
