@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libaicomp_kv.so")
 SOURCES = ["capi.hip", "kv_append.hip", "decode_generic.hip", "decode_mfma.hip", "prefill_mfma.hip",
-           "prefill_tiled.hip", "rope_append.hip", "sample.hip"]
+           "prefill_mfma_f32.hip", "prefill_tiled.hip", "rope_append.hip", "sample.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",

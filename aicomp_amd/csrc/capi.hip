@@ -31,6 +31,8 @@ int launch_kv_append(const void* key, const void* value, int64_t token_stride, i
 
 bool prefill_mfma_supported(const DecodeArgs& a, int max_q_len);
 int launch_prefill_mfma(const DecodeArgs& a, int max_q_len);
+bool prefill_mfma_f32_supported(const DecodeArgs& a, int max_q_len);
+int launch_prefill_mfma_f32(const DecodeArgs& a, int max_q_len);
 bool prefill_tiled_supported(const DecodeArgs& a, int max_q_len);
 int launch_prefill_tiled(const DecodeArgs& a, int max_q_len);
 
@@ -442,8 +444,10 @@ int aicomp_paged_prefill_attn(void* out, const void* query, const void* k_pool, 
     a.v_scale = kv_dtype == AICOMP_KV_FP8_E4M3 ? v_scale : nullptr;
     a.stream = (hipStream_t)stream;
     if (prefill_mfma_supported(a, max_q_len)) return launch_prefill_mfma(a, max_q_len);
-    // float32 models, head_dim 256, other block sizes: the tiled vector-ALU kernel (K/V staged in
-    // LDS once per 32 query rows)
+    // float32 models at head_dim 64 / 128: the float32 matrix instruction
+    if (prefill_mfma_f32_supported(a, max_q_len)) return launch_prefill_mfma_f32(a, max_q_len);
+    // head_dim 256, other block sizes: the tiled vector-ALU kernel (K/V staged in LDS once per 32
+    // query rows)
     if (prefill_tiled_supported(a, max_q_len)) return launch_prefill_tiled(a, max_q_len);
     // what is left (pools that cannot be read 16 bytes at a time): every query row as its own
     // unsplit attention problem over its causal prefix

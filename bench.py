@@ -510,12 +510,12 @@ def prefill_shapes_bench(dev, reps=20):
         t = e0.elapsed_time(e1) / reps * 1e-3
         flops = nseq * 4 * hq * d * (n * prior + n * (n + 1) / 2)
         f32 = qt == torch.float32
-        peak = 157.3 if f32 else MFMA_BF16_PEAK_TFLOPS          # fp32 vector / matrix peak, published
+        peak = 157.3 if f32 else MFMA_BF16_PEAK_TFLOPS          # fp32 matrix peak, published
         name = lambda t_: str(t_).replace("torch.", "")
         out.append({"chunks": nseq, "new_tokens": n, "prior": prior, "head_dim": d,
                     "q_dtype": name(qt), "kv_dtype": name(kvt), "us": round(t * 1e6, 1),
                     "TFLOPs": round(flops / t / 1e12, 1),
-                    "kernel": "paged_prefill_tiled_kernel" if f32 else "paged_prefill_mfma_kernel",
+                    "kernel": "paged_prefill_mfma_f32_kernel" if f32 else "paged_prefill_mfma_kernel",
                     "peak_TFLOPs": peak, "frac_mfma_peak": round(flops / t / 1e12 / peak, 4)})
         del k, v, q, o
         torch.cuda.empty_cache()

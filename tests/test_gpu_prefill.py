@@ -39,7 +39,7 @@ def build_case(device, priors, news, hq, hkv, d, bs=16, dtype=torch.bfloat16, kv
         v_pool = (vf / vs[None, :, None, None]).to(kv_dtype)
     else:
         k_pool, v_pool = kf.to(kv_dtype), vf.to(kv_dtype)
-        if poison and kv_dtype != torch.float32:
+        if poison and (kv_dtype != torch.float32 or poison == "all"):
             # every slot at or beyond a sequence's context is non-finite
             used = torch.zeros(nb * bs, dtype=torch.bool)
             for s, c in enumerate(ctx):
@@ -143,16 +143,47 @@ def test_prefill_fp32_and_other_shapes_use_the_generic_kernel(device):
 
 
 @pytest.mark.parametrize("hq,hkv,d,bs", [(8, 2, 128, 16), (4, 4, 64, 16), (6, 2, 128, 16), (16, 2, 64, 32),
-                                         (4, 1, 256, 16)])
-def test_prefill_fp32_tiled_kernel(device, hq, hkv, d, bs):
-    """float32 models (the reference's ``--dtype float32``) take the tiled vector kernel: a fresh
-    512-token prompt, a continuation across tile and block boundaries, ragged and one-token chunks,
-    groups of 1, 3 (one head per workgroup), 4 and 8; <= 1e-5 against the float64 oracle."""
+                                         (4, 1, 256, 16), (32, 8, 64, 16), (16, 1, 128, 16), (16, 2, 128, 16)])
+def test_prefill_fp32_kernels(device, hq, hkv, d, bs):
+    """float32 models (the reference's ``--dtype float32``) take the float32 matrix-instruction kernel
+    (head_dim 64 / 128, block 16) or the tiled vector kernel (the rest): a fresh 512-token prompt, a
+    continuation across tile and block boundaries, ragged and one-token chunks, groups of 1, 3 (one
+    head per workgroup), 4, 8 and 16; <= 1e-5 against the float64 oracle."""
     c = build_case(device, priors=[0, 300, 5, 0, 63, 31], news=[512, 130, 33, 1, 1, 70], hq=hq, hkv=hkv, d=d, bs=bs,
                    dtype=torch.float32, seed=d + bs)
     got = run(c, max_q_len=512)
     assert torch.isfinite(got).all()
     assert np.abs(to_f64(got) - oracle(c)).max() <= 1e-5
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (8, 8, 64), (3, 1, 128)])
+def test_prefill_fp32_matrix_kernel_ignores_everything_beyond_the_context(device, hq, hkv, d):
+    """float32 pools with NaN in every K slot and Inf in every V slot at or beyond a sequence's
+    context (tile tails, table padding): none of it may reach the output.  Priors and lengths put
+    the context end at every position of a 32-token tile's two blocks."""
+    c = build_case(device, priors=[0, 17, 31, 100, 3], news=[33, 16, 1, 61, 160], hq=hq, hkv=hkv, d=d,
+                   dtype=torch.float32, seed=7 + d, poison="all")
+    got = run(c, max_q_len=160)
+    assert torch.isfinite(got).all()
+    assert np.abs(to_f64(got) - oracle(c)).max() <= 1e-5
+
+
+def test_prefill_fp32_long_prompt_all_rows(device):
+    """A fresh 2048-token float32 prompt at the Llama-3 head shape (the bench's float32 shape): every
+    row within 1e-5 of the float64 oracle, and equal to torch's own is_causal=True float32 SDPA on
+    the gathered K/V to float32 round-off."""
+    n = 2048
+    c = build_case(device, priors=[0], news=[n], hq=32, hkv=8, d=128, dtype=torch.float32, seed=9)
+    got = run(c)
+    want = orc.paged_prefill_attn(raw(c["q"]), raw(c["k_pool"]), raw(c["v_pool"]), c["table"].cpu().numpy(), [n], [0, n],
+                                  c["scale"], "f32", "f32", gather=orc.gather_context_fast)
+    assert np.abs(to_f64(got) - want).max() <= 1e-5
+    blocks = c["table"][0, : n // 16].long()
+    k = c["k_pool"][blocks].permute(1, 0, 2, 3).reshape(8, n, 128)
+    v = c["v_pool"][blocks].permute(1, 0, 2, 3).reshape(8, n, 128)
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        c["q"].permute(1, 0, 2)[None], k.repeat_interleave(4, 0)[None], v.repeat_interleave(4, 0)[None], is_causal=True)
+    assert (ref[0].permute(1, 0, 2) - got).abs().max().item() <= 2e-5
 
 
 @pytest.mark.parametrize("dtype,kv_dtype,d,bs", [(torch.bfloat16, None, 256, 16), (torch.bfloat16, None, 128, 32),
