@@ -583,8 +583,8 @@ __device__ __forceinline__ int sk_tiles(int len, int max_blocks) {
 
 
 // PAIR: head_dim 64 as rows of token pairs (see paged_decode_mfma_kernel): a tile is 64 tokens in
-// four blocks, every head takes two B-operand columns (one per token parity), and a flush writes
-// one partial per column, of which only the 64 elements of the column's own token are kept.
+// four blocks, every head takes two B-operand columns (one per token parity), and a flush merges
+// the two columns of a head inside the wave and writes one partial of 64 floats per head.
 template <typename E, bool FP8, bool PAIR>
 __global__ void __launch_bounds__(256, 1)     // one workgroup per CU: a wave may use the whole register file
 streamk_decode_kernel(StreamKParams p) {
@@ -811,17 +811,38 @@ streamk_decode_kernel(StreamKParams p) {
         float lsum = st.lsum;
         lsum += __shfl_xor(lsum, 16);
         lsum += __shfl_xor(lsum, 32);
-        // PAIR: column (head, parity) keeps elements 64 * parity .. + 63 of its accumulator (its own token's
-        // half of the pair rows), i.e. the lanes with g4 / 2 == parity, as a partial of 64 floats
-        if (r16 < ncol && (!PAIR || (g4 >> 1) == (r16 & 1))) {
-            const int64_t slot = (int64_t)kvh * (p.waves_per_head + B) + part + seq;
-            float* dst = p.ws_acc + (slot * ncol + r16) * DQ + 32 * (PAIR ? (g4 & 1) : g4);
+        const int64_t slot = (int64_t)kvh * (p.waves_per_head + B) + part + seq;
+        if constexpr (PAIR) {
+            // Column (head, parity) holds its own token's half of the pair rows: parity 0 elements 0..63 of
+            // its accumulator (lanes g4 = 0, 1), parity 1 elements 64..127 (lanes g4 = 2, 3).  The two are
+            // partial softmaxes over the even and the odd tokens of the same segment: merged here, inside the
+            // wave, so that a flush writes ONE partial of 64 floats per head.  Lane (column 2h, g4 = a) takes
+            // the matching values of lane (column 2h + 1, g4 = a + 2), 33 lanes up.
+            const float m1 = __shfl_xor(st.m, 1), l1 = __shfl_xor(lsum, 1);
+            const float mm = fmaxf(st.m, m1);
+            const float f0 = exp2f(st.m - mm), f1 = exp2f(m1 - mm);
+            float mine[8][4];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) mine[j][i] = fmaf(f1, __shfl(st.O[j][i], lane + 33), f0 * st.O[j][i]);
+            if (r16 < ncol && (r16 & 1) == 0 && g4 < 2) {
+                float* dst = p.ws_acc + (slot * G + (r16 >> 1)) * DQ + 32 * g4;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    *(float4*)(dst + 8 * i) = make_float4(mine[0][i], mine[1][i], mine[2][i], mine[3][i]);
+                    *(float4*)(dst + 8 * i + 4) = make_float4(mine[4][i], mine[5][i], mine[6][i], mine[7][i]);
+                }
+                if (g4 == 0) *(float2*)(p.ws_ml + (slot * G + (r16 >> 1)) * 2) = make_float2(mm, f0 * lsum + f1 * l1);
+            }
+        } else if (r16 < ncol) {
+            float* dst = p.ws_acc + (slot * G + r16) * DQ + 32 * g4;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 *(float4*)(dst + 8 * i) = make_float4(st.O[0][i], st.O[1][i], st.O[2][i], st.O[3][i]);
                 *(float4*)(dst + 8 * i + 4) = make_float4(st.O[4][i], st.O[5][i], st.O[6][i], st.O[7][i]);
             }
-            if ((g4 & (PAIR ? 1 : 3)) == 0) *(float2*)(p.ws_ml + (slot * ncol + r16) * 2) = make_float2(st.m, lsum);
+            if (g4 == 0) *(float2*)(p.ws_ml + (slot * G + r16) * 2) = make_float2(st.m, lsum);
         }
         // the waves holding a row's first and last tile tell the merge kernel where its partials are
         if (lane == 0) {
@@ -845,66 +866,71 @@ streamk_decode_kernel(StreamKParams p) {
 // head of the group.  The row's partials sit in consecutive slots of its head's region,
 // head_slots * head + first + sequence .. + last + sequence (first / last part recorded by the
 // main kernel); their weights 2^(m_i - M) are computed once (one lane
-// per partial) and parked in LDS, then each lane accumulates two output dims with independent
-// loads.  With S = 1 (few partials per row, the usual batch) reductions are shuffles and there is
-// no barrier; with S > 1 (a handful of very long rows, hundreds of partials each) the waves of a
-// head take alternate groups of eight partials and add up through LDS.
+// per partial) and parked in LDS, then each lane accumulates its output dims (two at head_dim
+// 128, one at head_dim 64) with independent loads.  With S = 1 (few partials per row, the usual
+// batch) reductions are shuffles and there is no barrier; with S > 1 (a handful of very long rows,
+// hundreds of partials each) the waves of a head take alternate groups of eight partials and add
+// up through LDS.
 constexpr int RED_WGT = 256;       // weights parked in LDS per wave; rows with more partials recompute the rest
-template <typename E>
+template <typename E, int DQ>
 __global__ void __launch_bounds__(1024)
 streamk_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ ws_acc,
                       const float* __restrict__ ws_ml, const int* __restrict__ ws_rows,
                       const int32_t* __restrict__ context_lens, int hq, int hkv, int group,
                       const float* __restrict__ v_scale, int head_slots) {
+    constexpr int NV = DQ / 64;                            // output dims per lane
     const int kvh = blockIdx.x, seq = blockIdx.y, wv = threadIdx.x >> 6;
     const int S = (int)(blockDim.x >> 6) / group;          // waves per head
     const int h = wv / S, sub = wv % S;
     const int lane = threadIdx.x & 63;
     __shared__ float wgt_all[16][RED_WGT];
-    __shared__ float part[16][D];
+    __shared__ float part[16][DQ];
     float* wgt = wgt_all[wv];
     const int64_t row = (int64_t)seq * hkv + kvh;
-    uint16_t* o = out + ((int64_t)seq * hq + kvh * group + h) * D;
+    uint16_t* o = out + ((int64_t)seq * hq + kvh * group + h) * DQ;
     // the length and the row's record are requested together (the record of an empty row was never
     // written and is not used)
     const int ctx = context_lens[seq];
     const int first = ws_rows[2 * row], last = ws_rows[2 * row + 1];
     if (ctx <= 0) {                          // no tiles, no partials: the output row is zero (whole workgroup)
-        if (sub == 0) { o[lane] = 0; o[lane + 64] = 0; }
+        if (sub == 0) {
+#pragma unroll
+            for (int e = 0; e < NV; ++e) o[lane + 64 * e] = 0;
+        }
         return;
     }
     const int np = last - first + 1;
     const int64_t slot0 = (int64_t)kvh * head_slots + first + seq;       // the row's partials: slots slot0 .. slot0 + np - 1
     const float* ml = ws_ml + (slot0 * group + h) * 2;                  // partial i at ml[i * group * 2]
-    const float* acc = ws_acc + (slot0 * group + h) * D + lane;         // partial i at acc[i * group * D]
+    const float* acc = ws_acc + (slot0 * group + h) * DQ + lane;        // partial i at acc[i * group * DQ]
+    const int64_t stride = (int64_t)group * DQ;
     if (S == 1 && np <= 8) {
         // The usual batch: a handful of partials per row.  Their (max, sum) pairs and this lane's
-        // two output dims of each are requested in one go, so the kernel is two memory latencies
+        // output dims of each are requested in one go, so the kernel is two memory latencies
         // deep (record, then partials) instead of four.
-        const int64_t stride = (int64_t)group * D;
         float2 mlv[8];
-        float a[8], b[8];
+        float a[8][NV];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int i = min(u, np - 1);
             mlv[u] = *(const float2*)(ml + (int64_t)i * group * 2);
-            a[u] = acc[i * stride];
-            b[u] = acc[i * stride + 64];
+#pragma unroll
+            for (int e = 0; e < NV; ++e) a[u][e] = acc[i * stride + 64 * e];
         }
         float mx = NEG_BIG;
 #pragma unroll
         for (int u = 0; u < 8; ++u) mx = fmaxf(mx, mlv[u].x);           // repeats of the last partial change nothing
-        float den = 0.f, n0 = 0.f, n1 = 0.f;
+        float den = 0.f, num[NV] = {};
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const float f = u < np ? exp2f(mlv[u].x - mx) : 0.f;
             den = fmaf(f, mlv[u].y, den);
-            n0 = fmaf(f, a[u], n0);
-            n1 = fmaf(f, b[u], n1);
+#pragma unroll
+            for (int e = 0; e < NV; ++e) num[e] = fmaf(f, a[u][e], num[e]);
         }
         const float inv = den > 0.f ? (v_scale ? v_scale[kvh] : 1.f) / den : 0.f;
-        o[lane] = E::from_f32(n0 * inv);
-        o[lane + 64] = E::from_f32(n1 * inv);
+#pragma unroll
+        for (int e = 0; e < NV; ++e) o[lane + 64 * e] = E::from_f32(num[e] * inv);
         return;
     }
     // every wave of a head computes the row's max, denominator and weights for itself (np / 64 loads per lane)
@@ -921,77 +947,36 @@ streamk_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ ws_a
     }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) den += __shfl_xor(den, off);
-    const int64_t stride = (int64_t)group * D;
-    // eight partials (sixteen loads) in flight per step: the loop is pure load latency
-    float n0 = 0.f, n1 = 0.f;
+    // eight partials in flight per step: the loop is pure load latency
+    float num[NV] = {};
     for (int i0 = 8 * sub; i0 < np; i0 += 8 * S) {
-        float a[8], b[8];
+        float a[8][NV];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int i = min(i0 + u, np - 1);
-            a[u] = acc[i * stride];
-            b[u] = acc[i * stride + 64];
+#pragma unroll
+            for (int e = 0; e < NV; ++e) a[u][e] = acc[i * stride + 64 * e];
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int i = i0 + u;
             const float f = i >= np ? 0.f : (i < RED_WGT ? wgt[i] : exp2f(ml[(int64_t)i * group * 2] - mx));
-            n0 = fmaf(f, a[u], n0);
-            n1 = fmaf(f, b[u], n1);
+#pragma unroll
+            for (int e = 0; e < NV; ++e) num[e] = fmaf(f, a[u][e], num[e]);
         }
     }
     if (S > 1) {                             // workgroup-uniform
-        part[wv][lane] = n0; part[wv][lane + 64] = n1;
+#pragma unroll
+        for (int e = 0; e < NV; ++e) part[wv][lane + 64 * e] = num[e];
         __syncthreads();
         if (sub != 0) return;
-        for (int k = 1; k < S; ++k) { n0 += part[wv + k][lane]; n1 += part[wv + k][lane + 64]; }
+        for (int k = 1; k < S; ++k)
+#pragma unroll
+            for (int e = 0; e < NV; ++e) num[e] += part[wv + k][lane + 64 * e];
     }
     const float inv = den > 0.f ? (v_scale ? v_scale[kvh] : 1.f) / den : 0.f;
-    o[lane] = E::from_f32(n0 * inv);
-    o[lane + 64] = E::from_f32(n1 * inv);
-}
-
-// Merge for head_dim 64 (pair rows): a row's partials are np waves x two token parities, 64 floats
-// each; one wave per head, lane = output dim.  Entry e = (part e / 2, parity e % 2).
-template <typename E>
-__global__ void __launch_bounds__(512)
-streamk_reduce_pair_kernel(uint16_t* __restrict__ out, const float* __restrict__ ws_acc,
-                           const float* __restrict__ ws_ml, const int* __restrict__ ws_rows,
-                           const int32_t* __restrict__ context_lens, int hq, int hkv, int group,
-                           const float* __restrict__ v_scale, int head_slots) {
-    const int kvh = blockIdx.x, seq = blockIdx.y, h = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int ncol = 2 * group;
-    const int64_t row = (int64_t)seq * hkv + kvh;
-    uint16_t* o = out + ((int64_t)seq * hq + kvh * group + h) * 64;
-    const int ctx = context_lens[seq];
-    const int first = ws_rows[2 * row], last = ws_rows[2 * row + 1];
-    if (ctx <= 0) { o[lane] = 0; return; }
-    const int ne = 2 * (last - first + 1);
-    const int64_t col0 = ((int64_t)kvh * head_slots + first + seq) * ncol + 2 * h;     // entry e: column col0 + (e / 2) * ncol + e % 2
-    auto col = [&](int e) { return col0 + (int64_t)(e >> 1) * ncol + (e & 1); };
-    float mx = NEG_BIG;
-    for (int e = lane; e < ne; e += 64) mx = fmaxf(mx, ws_ml[col(e) * 2]);
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-    float den = 0.f, num = 0.f;
-    for (int e0 = 0; e0 < ne; e0 += 8) {                     // eight entries in flight per step
-        float2 ml[8];
-        float a[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int64_t c = col(min(e0 + u, ne - 1));
-            ml[u] = *(const float2*)(ws_ml + c * 2);
-            a[u] = ws_acc[c * 64 + lane];
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const float f = e0 + u < ne ? exp2f(ml[u].x - mx) : 0.f;
-            den = fmaf(f, ml[u].y, den);
-            num = fmaf(f, a[u], num);
-        }
-    }
-    const float inv = den > 0.f ? (v_scale ? v_scale[kvh] : 1.f) / den : 0.f;
-    o[lane] = E::from_f32(num * inv);
+    for (int e = 0; e < NV; ++e) o[lane + 64 * e] = E::from_f32(num[e] * inv);
 }
 
 }  // namespace
@@ -1014,10 +999,10 @@ bool decode_streamk_supported(const DecodeArgs& a) {
     return decode_mfma_supported(a) && a.rows <= SK_MAX_SEQS && a.hkv <= 256;
 }
 
-// per slot one partial per B-operand column: G columns of D + 2 floats, or 2 G columns of 64 + 2 (head_dim 64)
+// per slot one partial per head: G x (head_dim + 2) floats
 size_t decode_streamk_workspace_bytes(int64_t rows, int hq, int hkv, int d) {
     const int64_t slots = SK_MAX_WAVES + rows * hkv;
-    const int ncol = d == 64 ? 2 * (hq / hkv) : hq / hkv;
+    const int ncol = hq / hkv;
     return (size_t)slots * ncol * (size_t)(d + 2) * sizeof(float) + (size_t)rows * hkv * 2 * sizeof(int);
 }
 
@@ -1052,7 +1037,7 @@ int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
     p.num_waves = wgs * NWAVES;
     p.waves_per_head = p.num_waves / a.hkv;
     const bool pair = a.d == 64;
-    const int ncol = pair ? 2 * group : group;
+    const int ncol = group;
     p.ws_acc = (float*)workspace;
     p.ws_ml = p.ws_acc + slots * ncol * a.d;
     p.ws_rows = (int*)(p.ws_ml + slots * ncol * 2);
@@ -1068,29 +1053,16 @@ int launch_decode_streamk(const DecodeArgs& a, void* workspace) {
     else { if (f16) AICOMP_LAUNCH_SK(F16Fmt, false); else AICOMP_LAUNCH_SK(Bf16Fmt, false); }
 #undef AICOMP_LAUNCH_SK
     AICOMP_HIP_LAUNCH_CHECK();
-    if (pair) {
-        if (f16)
-            hipLaunchKernelGGL(streamk_reduce_pair_kernel<F16Fmt>, dim3(a.hkv, (unsigned)a.rows), dim3(64 * group), 0,
-                               a.stream, (uint16_t*)a.out, p.ws_acc, p.ws_ml, p.ws_rows, a.context_lens, a.hq, a.hkv,
-                               group, a.v_scale, p.waves_per_head + (int)a.rows);
-        else
-            hipLaunchKernelGGL(streamk_reduce_pair_kernel<Bf16Fmt>, dim3(a.hkv, (unsigned)a.rows), dim3(64 * group), 0,
-                               a.stream, (uint16_t*)a.out, p.ws_acc, p.ws_ml, p.ws_rows, a.context_lens, a.hq, a.hkv,
-                               group, a.v_scale, p.waves_per_head + (int)a.rows);
-        AICOMP_HIP_LAUNCH_CHECK();
-        return AICOMP_KV_OK;
-    }
     // waves per head in the merge: one, unless rows are few and long (many partials per row)
     const int64_t per_row = (int64_t)p.waves_per_head / a.rows + 2;
     const int sub = per_row > 8 ? 16 / group : 1;
-    if (f16)
-        hipLaunchKernelGGL(streamk_reduce_kernel<F16Fmt>, dim3(a.hkv, (unsigned)a.rows), dim3(64 * group * sub), 0,
-                           a.stream, (uint16_t*)a.out, p.ws_acc, p.ws_ml, p.ws_rows, a.context_lens, a.hq, a.hkv,
-                           group, a.v_scale, p.waves_per_head + (int)a.rows);
-    else
-        hipLaunchKernelGGL(streamk_reduce_kernel<Bf16Fmt>, dim3(a.hkv, (unsigned)a.rows), dim3(64 * group * sub), 0,
-                           a.stream, (uint16_t*)a.out, p.ws_acc, p.ws_ml, p.ws_rows, a.context_lens, a.hq, a.hkv,
-                           group, a.v_scale, p.waves_per_head + (int)a.rows);
+#define AICOMP_LAUNCH_RED(E, DQ)                                                                                  \
+    hipLaunchKernelGGL((streamk_reduce_kernel<E, DQ>), dim3(a.hkv, (unsigned)a.rows), dim3(64 * group * sub), 0,  \
+                       a.stream, (uint16_t*)a.out, p.ws_acc, p.ws_ml, p.ws_rows, a.context_lens, a.hq, a.hkv,     \
+                       group, a.v_scale, p.waves_per_head + (int)a.rows)
+    if (pair) { if (f16) AICOMP_LAUNCH_RED(F16Fmt, 64); else AICOMP_LAUNCH_RED(Bf16Fmt, 64); }
+    else { if (f16) AICOMP_LAUNCH_RED(F16Fmt, 128); else AICOMP_LAUNCH_RED(Bf16Fmt, 128); }
+#undef AICOMP_LAUNCH_RED
     AICOMP_HIP_LAUNCH_CHECK();
     return AICOMP_KV_OK;
 }

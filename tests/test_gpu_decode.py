@@ -471,7 +471,7 @@ def test_balanced_schedule_records_the_parts_the_host_model_predicts(hkv, group,
     dev = torch.device("cuda:0")
     g = torch.Generator().manual_seed(11 + hkv)
     B, hq = 37, hkv * group
-    tile, ncol = (64, 2 * group) if D == 64 else (32, group)       # head_dim 64: pair rows, two columns per head
+    tile, ncol = (64 if D == 64 else 32), group                    # head_dim 64: pair rows; one partial per head either way
     lens = torch.randint(1, 3000, (B,), generator=g).tolist()
     lens[3] = 0; lens[4] = 0; lens[20] = 1; lens[36] = 33
     need = [max(1, math.ceil(c / 16)) for c in lens]
