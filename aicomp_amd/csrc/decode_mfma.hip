@@ -24,8 +24,9 @@
 //              each global_load_dwordx4 of a wave reads 1 KB = 4 whole rows,
 //              lane l -> row l/16, 16-byte chunk l%16.  One table lookup per
 //              block, wave-uniform (scalar).
-// K            staged through a wave-private LDS tile (row stride 272 B, so the
-//              16 rows a quarter-wave reads hit distinct banks) and read back
+// K            staged through a wave-private LDS tile (unpadded 256-byte rows whose
+//              16-byte chunks are permuted by a function of the row, so that the
+//              operand reads run at the full LDS rate) and read back
 //              as the A operand of  S^T = K Q^T  (v_mfma_f32_16x16x32_bf16 / _f16),
 //              the G query heads (padded to 16 columns) sharing every K tile.
 // V            never touches LDS.  Lane (c = l%16, q = l/16) of load i holds
@@ -51,8 +52,8 @@ constexpr int D = 128;
 constexpr int BS = 16;
 constexpr int TILE = 32;               // tokens per wave iteration (two blocks)
 constexpr int NWAVES = 4;
-constexpr int KROW = 272;              // LDS row stride in bytes (256 + 16 pad)
-constexpr int KTILE_BYTES = TILE * KROW;   // 8704 per wave
+constexpr int KROW = 256;              // LDS row stride in bytes: unpadded, 16-byte chunks swizzled (below)
+constexpr int KTILE_BYTES = TILE * KROW;   // 8192 per wave
 constexpr float NEG_BIG = -1.0e30f;
 constexpr int SK_MAX_WAVES = 4096;     // balanced schedule: at most 1024 workgroups of 4 waves
 
@@ -155,6 +156,31 @@ __device__ __forceinline__ int64_t clamp_block(int b, int64_t num_blocks) {
     return b < 0 ? 0 : (b >= num_blocks ? num_blocks - 1 : (int64_t)b);
 }
 
+// Where a lane writes and reads the wave's K tile.  Chunk slot s of tile row r holds the row's
+// chunk s ^ swz(r), swz(r) = ((r / 4) % 4) | ((r % 4) * 4): the operand read below then has every
+// four consecutive lanes in one aligned 64-byte segment and each half-wave spread evenly over the
+// four segments of a 256-byte bank line, which is what the LDS needs to deliver 256 bytes per
+// clock (rows padded to 272 bytes are free of bank collisions among the sixteen lanes of an MFMA
+// row group, yet run at half that rate: a quarter of the LDS cycles were conflict cycles).
+//   write  load i of lane (q = lane / 16, c = lane % 16) is row 4 i + q, chunk c:
+//          swz = (i % 4) | (q * 4), so four distinct offsets, picked by i % 4
+//   read   sub-tile a, k-step s, lane (r16, g4): row 16 a + 4 (r16 % 4) + r16 / 4, chunk 4 s + g4:
+//          swz of that row is r16 itself, so the slot is (4 s + g4) ^ r16
+struct KTileOffsets {
+    int wr[4];
+    int rd[4];
+};
+__device__ __forceinline__ KTileOffsets k_tile_offsets(int lane) {
+    const int r16 = lane & 15, g4 = lane >> 4;
+    KTileOffsets o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        o.wr[k] = g4 * KROW + ((r16 ^ (k | (g4 << 2))) << 4);
+        o.rd[k] = (4 * (r16 & 3) + (r16 >> 2)) * KROW + (((4 * k + g4) ^ r16) << 4);
+    }
+    return o;
+}
+
 // Per-wave running state of the online softmax and the output accumulators.
 struct WaveState {
     float m, lsum;
@@ -168,8 +194,8 @@ struct WaveState {
 // + 2r + 1, the B-operand columns are (head, parity) pairs, column c scoring token 2r + (c & 1).
 template <typename E, bool FP8, bool NEXT, bool MASK, bool PAIR = false>
 __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, TileRegs<FP8>& vr,
-                                             const uint4 (&qf)[4], unsigned char* kt, int wr_off,
-                                             int rd_off, const void* k_pool, const void* v_pool,
+                                             const uint4 (&qf)[4], unsigned char* kt, const KTileOffsets& ko,
+                                             const void* k_pool, const void* v_pool,
                                              int64_t nb0, int64_t nb1, int hkv, int kvh_next, int lane,
                                              int g4, int tile_start, int end, float cmul,
                                              int64_t nb2 = 0, int64_t nb3 = 0) {
@@ -180,7 +206,7 @@ __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, T
         // PAIR: a row's two tokens share every dot product (the query column is zero over the other
         // token's half), so a token beyond the context must not leave non-finite values in the row
         if (PAIR && MASK && tile_start + 2 * (4 * i + g4) + ((lane & 15) >> 3) >= end) kk = make_uint4(0, 0, 0, 0);
-        *(uint4*)(kt + wr_off + i * 4 * KROW) = kk;
+        *(uint4*)(kt + ko.wr[i & 3] + i * 4 * KROW) = kk;
     }
     if (NEXT) {
         if constexpr (PAIR) load_tile_pair<FP8>(kr, k_pool, nb0, nb1, nb2, nb3, hkv, kvh_next, lane);
@@ -191,8 +217,8 @@ __device__ __forceinline__ void process_tile(WaveState& st, TileRegs<FP8>& kr, T
     f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-        const uint4 a0 = *(const uint4*)(kt + rd_off + s * 64);
-        const uint4 a1 = *(const uint4*)(kt + rd_off + 16 * KROW + s * 64);
+        const uint4 a0 = *(const uint4*)(kt + ko.rd[s]);
+        const uint4 a1 = *(const uint4*)(kt + ko.rd[s] + 16 * KROW);
         s0 = E::mfma(a0, qf[s], s0);
         s1 = E::mfma(a1, qf[s], s1);
     }
@@ -402,10 +428,7 @@ paged_decode_mfma_kernel(MfmaParams p) {
             bb[j] = clamp_block(__builtin_amdgcn_readlane(tab, i0 + j - tab_first), p.num_blocks);
     };
 
-    // LDS addresses: write row = 4i + lane/16, chunk lane%16;
-    // read (sub-tile a, k-step s): row 16a + 4*(r16%4) + r16/4, chunk 4s + g4
-    const int wr_off = (lane >> 4) * KROW + (lane & 15) * 16;
-    const int rd_off = (4 * (r16 & 3) + (r16 >> 2)) * KROW + g4 * 16;
+    const KTileOffsets ko = k_tile_offsets(lane);
 
     if (w < ntiles) {
         TileRegs<FP8> kr, vr;
@@ -423,7 +446,7 @@ paged_decode_mfma_kernel(MfmaParams p) {
         int tt = w;
         for (; tt + NWAVES < ntiles; tt += NWAVES) {      // steady state: never the partition's last tile
             tile_blocks(tt + NWAVES);
-            process_tile<E, FP8, true, false, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, bb[0],
+            process_tile<E, FP8, true, false, PAIR>(st, kr, vr, qf, kt, ko, p.k_pool, p.v_pool, bb[0],
                                                  bb[1], p.hkv, kvh, lane, g4, start + tt * TT, end, cmul,
                                                  bb[2], bb[3]);
         }
@@ -439,10 +462,10 @@ paged_decode_mfma_kernel(MfmaParams p) {
                 inject_new_row_grid<E, FP8, PAIR>(kr, vr, p, seq, kvh, lane, tile_start, len, bb);
         }
         if (tile_start + TT > end)
-            process_tile<E, FP8, false, true, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
+            process_tile<E, FP8, false, true, PAIR>(st, kr, vr, qf, kt, ko, p.k_pool, p.v_pool, 0, 0,
                                                  p.hkv, kvh, lane, g4, tile_start, end, cmul);
         else
-            process_tile<E, FP8, false, false, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
+            process_tile<E, FP8, false, false, PAIR>(st, kr, vr, qf, kt, ko, p.k_pool, p.v_pool, 0, 0,
                                                   p.hkv, kvh, lane, g4, tile_start, end, cmul);
     }
     const float m = st.m;
@@ -452,7 +475,7 @@ paged_decode_mfma_kernel(MfmaParams p) {
     // ---- wave result: lane (column r16, g4) holds O^T[element 32*g4 + 8*i + j][column] in O[j][i]
     lsum += __shfl_xor(lsum, 16);
     lsum += __shfl_xor(lsum, 32);
-    float* osm = (float*)kt;        // this wave's own K tile region, 16 columns * 128 floats <= 8704 bytes
+    float* osm = (float*)kt;        // this wave's own K tile region, 16 columns * 128 floats = 8192 bytes, the whole tile
     if (r16 < ncol) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -672,8 +695,7 @@ streamk_decode_kernel(StreamKParams p) {
     int kvh = __builtin_amdgcn_readfirstlane(kvh_mine);
     int t = __builtin_amdgcn_readfirstlane((int)(g0 - prefix[seq]));
 
-    const int wr_off = (lane >> 4) * KROW + (lane & 15) * 16;
-    const int rd_off = (4 * (r16 & 3) + (r16 >> 2)) * KROW + g4 * 16;
+    const KTileOffsets ko = k_tile_offsets(lane);
 
     // ---- segments.  A segment is the part of one (sequence, KV head) row that falls into this
     // wave's tile range.  The next segment's query rows and table slice are requested while the
@@ -776,7 +798,7 @@ streamk_decode_kernel(StreamKParams p) {
         int k = 0;
         for (; k + 1 < nt; ++k) {
             tile_blocks(k + 1, bb);
-            process_tile<E, FP8, true, false, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, bb[0], bb[1],
+            process_tile<E, FP8, true, false, PAIR>(st, kr, vr, qf, kt, ko, p.k_pool, p.v_pool, bb[0], bb[1],
                                                     p.hkv, kvh, lane, g4, (t + k) * TT, len, cmul, bb[2], bb[3]);
         }
         const int tile_start = (t + k) * TT;
@@ -800,10 +822,10 @@ streamk_decode_kernel(StreamKParams p) {
             q_operand(qraw, qn);
             tab_ready = tabn;
             slice_blocks(tab_ready, 0, bb);
-            process_tile<E, FP8, true, true, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, bb[0], bb[1],
+            process_tile<E, FP8, true, true, PAIR>(st, kr, vr, qf, kt, ko, p.k_pool, p.v_pool, bb[0], bb[1],
                                                    p.hkv, nkvh, lane, g4, tile_start, len, cmul, bb[2], bb[3]);
         } else {
-            process_tile<E, FP8, false, true, PAIR>(st, kr, vr, qf, kt, wr_off, rd_off, p.k_pool, p.v_pool, 0, 0,
+            process_tile<E, FP8, false, true, PAIR>(st, kr, vr, qf, kt, ko, p.k_pool, p.v_pool, 0, 0,
                                                     p.hkv, kvh, lane, g4, tile_start, len, cmul);
         }
 
