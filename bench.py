@@ -367,6 +367,92 @@ def small_batch_decode_bench(dev):
     return {"shape": "32 query / 8 KV heads, head_dim 64, bf16", "calls": out_rows}
 
 
+def mixed_step_graph(dev, two_streams):
+    """The chunked-prefill mixed step (4 chunks of 512 tokens + 60 decode sequences) recorded into a
+    HIP graph of three steps over three K/V pools, and a function that replays it.  Serial: append of
+    the chunk rows, prefill, fused append + decode, one after the other.  Two streams: the decode call
+    is launched first on one stream and the append + prefill on a second one, forked from and joined
+    to the step's stream with events, so that the hardware may run them side by side (a graph keeps
+    the host's stream and event calls out of the figure)."""
+    import torch
+    from aicomp_amd import ops, workloads
+    w = workloads.make_workload("chunked_prefill_mixed", device=dev)
+    npre = w.num_prefill_seqs
+    T = int(w.cu_q_lens[npre])
+    qd, btd, cld = w.query[T:].contiguous(), w.block_table[npre:].contiguous(), w.context_lens[npre:].contiguous()
+    qp, btp, clp = w.query[:T].contiguous(), w.block_table[:npre].contiguous(), w.context_lens[:npre].contiguous()
+    cup = w.cu_q_lens[:npre + 1].contiguous()
+    outd, outp = torch.empty_like(qd), torch.empty_like(qp)
+    nkd, nvd = w.new_key[T:].contiguous(), w.new_value[T:].contiguous()
+    nkp, nvp, smp = w.new_key[:T].contiguous(), w.new_value[:T].contiguous(), w.slot_mapping[:T].contiguous()
+    pools = [(w.k_pool, w.v_pool)] + [(w.k_pool.clone(), w.v_pool.clone()) for _ in range(2)]
+    s = w.shape
+    ws = torch.empty(ops.decode_workspace_bytes(len(w.ctx_list) - npre, s.num_q_heads, s.num_kv_heads, s.head_dim, s.block_size,
+                                                btd.shape[1], qd.dtype, w.k_pool.dtype), dtype=torch.uint8, device=dev)
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+
+    def decode(kp, vp):
+        ops.paged_decode_attn(outd, qd, kp, vp, btd, cld, w.scale, workspace=ws, new_key=nkd, new_value=nvd)
+
+    def prefill(kp, vp):
+        ops.kv_append(nkp, nvp, kp, vp, smp)
+        ops.paged_prefill_attn(outp, qp, kp, vp, btp, clp, cup, w.scale, max_q_len=max(w.new_list[:npre]))
+
+    def step(i):
+        kp, vp = pools[i % 3]
+        if not two_streams:
+            prefill(kp, vp)
+            decode(kp, vp)
+            return
+        main = torch.cuda.current_stream()
+        fork = torch.cuda.Event()
+        fork.record(main)
+        sa.wait_event(fork)
+        sb.wait_event(fork)
+        with torch.cuda.stream(sa):
+            decode(kp, vp)
+        with torch.cuda.stream(sb):
+            prefill(kp, vp)
+        ja, jb = torch.cuda.Event(), torch.cuda.Event()
+        ja.record(sa)
+        jb.record(sb)
+        main.wait_event(ja)
+        main.wait_event(jb)
+
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for i in range(3):
+            step(i)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(3):
+                step(i)
+    torch.cuda.synchronize()
+    return graph.replay, ("decode on one stream, append + prefill on another" if two_streams else "one stream")
+
+
+def mixed_step_bench(dev, reps=40):
+    """Mixed step replayed from a graph, one stream against two (see mixed_step_graph): us per step."""
+    import torch
+    res = {}
+    for name, two in (("one_stream_us", False), ("two_streams_us", True)):
+        fn, _ = mixed_step_graph(dev, two)
+        for _ in range(5):
+            fn()
+        e0, e1 = _events(2)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        res[name] = round(e0.elapsed_time(e1) / (3 * reps) * 1e3, 1)
+        del fn
+        torch.cuda.empty_cache()
+    res["note"] = ("graph replays of 3 steps over 3 pools; two streams: decode launched first, append + prefill beside it, "
+                   "forked and joined with events")
+    return res
+
+
 def host_cost_bench(dev):
     """Host time of ONE decode call of the drop-in operator at the size the reference's own engine
     runs (batch 1, Llama-3.2-1B heads: 32 / 8, head_dim 64, bf16, K/V arriving expanded by
@@ -594,6 +680,13 @@ def profile_target(which, steps, warmup, dev, settle_ms=30.0):
         how = drive(lambda: ops.sample_tokens(logits, 0.8, 50, 0.9, uniforms=u))
         print(f"sample: {how}, over [64, 128256] fp32 logits, temperature 0.8, top-k 50, top-p 0.9")
         return
+    if which in ("mixed_serial", "mixed_streams"):
+        fn, how = mixed_step_graph(dev, two_streams=which == "mixed_streams")
+        for _ in range(warmup + steps):
+            fn()
+        torch.cuda.synchronize()
+        print(f"{which}: {warmup + steps} replays of a graph of 3 mixed steps ({how})")
+        return
     if which == "prefill_long":
         # one fresh prompt of 8192 tokens at the Llama-3-8B head shape (a row of prefill_other_shapes)
         import math
@@ -739,7 +832,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
-    ap.add_argument("--only", choices=["decode", "append", "copy", "prefill", "prefill_long", "decode_fp8", "decode_long", "decode_d64", "rope", "sample"],
+    ap.add_argument("--only", choices=["decode", "append", "copy", "prefill", "prefill_long", "decode_fp8", "decode_long", "decode_d64", "rope", "sample",
+                             "mixed_serial", "mixed_streams"],
                     help="profiling target: launch just this kernel --steps times (no JSON line)")
     ap.add_argument("--settle-ms", type=float, default=30.0,
                     help="with --only: untimed launches for this long before the timed ones")
@@ -796,6 +890,7 @@ def main():
         "sampler": sampler_bench(dev),
         "decode_small_batch": small_batch_decode_bench(dev),
         "operator_host_cost": host_cost_bench(dev),
+        "mixed_step_streams": mixed_step_bench(dev),
         "prefill_other_shapes": prefill_shapes_bench(dev),
     }
     if not args.no_cpu:
