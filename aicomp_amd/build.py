@@ -72,6 +72,28 @@ def build_torch_ops(verbose: bool = True) -> str:
     return TORCH_LIB
 
 
+def build_fast_call(verbose: bool = True) -> str:
+    """Compile csrc/fast_call.cpp into the CPython module aicomp_amd._aicomp_fast: the operator's
+    decode call as one METH_FASTCALL function over the same library (host code only)."""
+    import sysconfig
+    import torch
+    from torch.utils import cpp_extension as ce
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    out = os.path.join(HERE, "_aicomp_fast" + sysconfig.get_config_var("EXT_SUFFIX"))
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1",
+           "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={int(torch.compiled_with_cxx11_abi())}",
+           f"-I{sysconfig.get_paths()['include']}", *[f"-I{d}" for d in ce.include_paths()], "-I/opt/rocm/include",
+           os.path.join(CSRC, "fast_call.cpp"), "-o", out, f"-L{tlib}", "-ltorch", "-ltorch_cpu", "-lc10",
+           "-ltorch_hip", "-lc10_hip", "-ltorch_python", f"-L{HERE}", "-laicomp_kv", "-Wl,-rpath,$ORIGIN",
+           f"-Wl,-rpath,{tlib}"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"compiling fast_call.cpp failed:\n{r.stdout}\n{r.stderr}")
+    if verbose:
+        print(f"built {out}")
+    return out
+
+
 def build_host_example(verbose: bool = True) -> str:
     """Compile tests/cabi_host.cpp, a C++ program that links the library directly (no Python, no
     torch): the boundary as a C or C++ host sees it."""
@@ -91,5 +113,6 @@ def build_host_example(verbose: bool = True) -> str:
 if __name__ == "__main__":
     build()
     build_torch_ops()
+    build_fast_call()
     build_host_example()
     sys.exit(0)

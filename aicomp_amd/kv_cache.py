@@ -46,13 +46,21 @@ from . import _lib, ops
 
 BLOCK_SIZE = 16
 
-# The decode step as one registered PyTorch operator (a third of the host time of the ctypes
-# route at batch 1).  Both routes end in the same C entry point of the HIP library; the ctypes
-# one remains for device-side positions and for installations without the registration library.
+# Host routes of a decode step into the HIP library, leanest first.  All three end in the same C
+# entry point (aicomp_paged_decode_attn_append); they differ in host time per call, which at
+# batch 1 is step time: "fast", a CPython function over a per-layer handle (csrc/fast_call.cpp);
+# "torch_op", the registered operator torch.ops.mi355_kv.decode_step (csrc/torch_ops.cpp);
+# "ctypes", which remains for device-side positions and for installations where the two host
+# libraries were not built.
+try:
+    from . import _aicomp_fast as _FAST
+except ImportError:
+    _FAST = None
 try:
     _TORCH_DECODE = _lib.torch_ops().decode_step.default
 except _lib.LibraryMissing:
     _TORCH_DECODE = None
+_route = "fast" if _FAST is not None else ("torch_op" if _TORCH_DECODE is not None else "ctypes")
 
 
 def _detect_group(key: torch.Tensor) -> int:
@@ -87,6 +95,7 @@ class _PagedLayer:
                  dtype: torch.dtype, device: torch.device, block_size: int = BLOCK_SIZE):
         self.batch, self.kv_heads, self.head_dim = batch, kv_heads, head_dim
         self.default_scale = 1.0 / math.sqrt(head_dim)
+        self.dtype = dtype
         self.max_seq_len, self.block_size = max_seq_len, block_size
         self.blocks_per_seq = max(1, math.ceil(max_seq_len / block_size))
         nb = batch * self.blocks_per_seq
@@ -106,6 +115,11 @@ class _PagedLayer:
         # replayed from a HIP graph (a replay runs no host code, so it cannot pick another row)
         self.live_ctx = torch.zeros(batch, dtype=torch.int32, device=device)
         self._ctx_base, self._ctx_pitch = self.ctx_rows.data_ptr(), self.ctx_rows.stride(0) * 4
+        # the static tensors, checked once, behind a handle for the lean decode call (pools of the
+        # operator's own element types; the handle keeps the tensors alive)
+        self._fast = None
+        if _FAST is not None and self.k_pool.is_cuda and dtype in (torch.float32, torch.bfloat16, torch.float16):
+            self._fast = _FAST.layer(self.k_pool, self.v_pool, self.block_table, self.ctx_rows)
         self._decode: Dict[tuple, ops.PreparedDecode] = {}
         self.cu_q_lens = torch.zeros(batch + 1, dtype=torch.int32, device=device)
         self._cu_n = -1
@@ -132,11 +146,13 @@ class _PagedLayer:
         key/value ``[B, H, 1, D]`` written at position pos.  With ``live`` the position is the
         device-side counter ``live_ctx`` (advanced here by a one-element-per-sequence kernel), so
         the step can be captured into a HIP graph and replayed."""
-        if not live and _TORCH_DECODE is not None:
-            # one dispatch through torch.ops.mi355_kv.decode_step: checks, output allocation,
-            # current stream and the fused append + decode call all happen in C++
-            return _TORCH_DECODE(query, key, value, self.k_pool, self.v_pool, self.block_table, self.ctx_rows, pos,
-                                 group, scale, None)
+        if not live and _route != "ctypes":
+            # checks, output allocation, current stream and the fused append + decode call all in C++
+            if _route == "fast" and self._fast is not None:
+                return _FAST.decode_step(self._fast, query, key, value, pos, group, scale)
+            if _TORCH_DECODE is not None:
+                return _TORCH_DECODE(query, key, value, self.k_pool, self.v_pool, self.block_table, self.ctx_rows,
+                                     pos, group, scale, None)
         Hq = query.shape[1]
         call = self._decode.get((Hq, query.dtype, scale))
         if call is None:
@@ -517,16 +533,16 @@ class CachedScaledDotProductAttention(nn.Module):
                 attn_mask: Optional[torch.Tensor] = None, dropout_p: float = 0.0,
                 is_causal: bool = False, **kwargs) -> torch.Tensor:
         # decode step on the operator's own cache, the call a generation loop makes once per layer
-        # and token: straight to the registered operator (checks, output, stream and launch in C++)
+        # and token: straight to the lean C++ entry (checks, output, stream and launch in one call)
         store = self._store
-        if (store is not None and self._enabled and self.kv_manager is None and not self._device_positions
-                and _TORCH_DECODE is not None and dropout_p == 0.0 and query.dim() == 4 and query.shape[2] == 1
-                and key.dtype == store.k_pool.dtype):
+        if (store is not None and store._fast is not None and _route == "fast" and self._enabled
+                and self.kv_manager is None and not self._device_positions and dropout_p == 0.0
+                and query.dim() == 4 and query.shape[2] == 1 and key.dtype == store.dtype):
             pos = self.cache_pos
             if pos < self.max_seq_len:
-                scale = kwargs.get("scale")
-                out = _TORCH_DECODE(query, key, value, store.k_pool, store.v_pool, store.block_table, store.ctx_rows,
-                                    pos, self._group, store.default_scale if scale is None else float(scale), None)
+                out = _FAST.decode_step(store._fast, query, key, value, pos, self._group,
+                                        store.default_scale if not kwargs or kwargs.get("scale") is None
+                                        else float(kwargs["scale"]))
                 self.cache_pos = pos + 1
                 return out
         if not self._enabled:

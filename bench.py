@@ -459,18 +459,20 @@ def host_cost_bench(dev):
     repeat_kv): the Python thread's time per call, timed over 1000 calls without a synchronisation
     inside (the position is set back before every call, so each call sees the stated context).
     At 600 cached tokens the call is one launch (whole rows), at 1500 two (256-token partitions and
-    their merge).  Through the registered operator (torch.ops.mi355_kv.decode_step) and through the
-    ctypes binding of the same C entry point."""
+    their merge).  Through each host route to the same C entry point: the CPython function over a
+    per-layer handle (the one the operator takes), the registered operator
+    (torch.ops.mi355_kv.decode_step) and the ctypes binding."""
     import torch
     from aicomp_amd import kv_cache as akv
     B, hq, g, d = 1, 32, 4, 64
     hkv = hq // g
     mk = lambda n, h: torch.randn(B, h, n, d, device=dev).to(torch.bfloat16)
     res = {"shape": "batch 1, 32 query / 8 KV heads (K/V expanded to 32), head_dim 64, bf16"}
-    for name, route in (("torch_op", akv._TORCH_DECODE), ("ctypes", None)):
-        if name == "torch_op" and route is None:
+    available = {"fast": akv._FAST is not None, "torch_op": akv._TORCH_DECODE is not None, "ctypes": True}
+    for name in ("fast", "torch_op", "ctypes"):
+        if not available[name]:
             continue
-        saved, akv._TORCH_DECODE = akv._TORCH_DECODE, route
+        saved, akv._route = akv._route, name
         try:
             op = akv.CachedScaledDotProductAttention(0, 2048, num_kv_groups=g)
             op.enable()
@@ -493,8 +495,9 @@ def host_cost_bench(dev):
                     best = host if best is None else min(best, host)
                 res[f"host_us_per_call_{name}_ctx{ctx}"] = round(best * 1e6, 2)
         finally:
-            akv._TORCH_DECODE = saved
-    res["host_us_per_call"] = res.get("host_us_per_call_torch_op_ctx600", res.get("host_us_per_call_ctypes_ctx600"))
+            akv._route = saved
+    res["route_in_use"] = akv._route
+    res["host_us_per_call"] = res[f"host_us_per_call_{akv._route}_ctx600"]
     return res
 
 

@@ -59,13 +59,15 @@ def decode_routing(request):
     ops.set_small_decode_tokens(prev)
 
 
-@pytest.fixture(params=["torch_op", "ctypes"])
+@pytest.fixture(params=["fast", "torch_op", "ctypes"])
 def host_route(request, monkeypatch):
-    """The two host routes of the drop-in operator's decode step into the HIP library: the
-    registered PyTorch operator (torch.ops.mi355_kv.decode_step) and the ctypes binding."""
+    """The host routes of the drop-in operator's decode step into the HIP library: the CPython
+    function over a per-layer handle (aicomp_amd._aicomp_fast), the registered PyTorch operator
+    (torch.ops.mi355_kv.decode_step) and the ctypes binding."""
     from aicomp_amd import kv_cache as akv
-    if request.param == "ctypes":
-        monkeypatch.setattr(akv, "_TORCH_DECODE", None)
-    else:
+    if request.param == "fast":
+        assert akv._FAST is not None, "aicomp_amd/_aicomp_fast is not built"
+    elif request.param == "torch_op":
         assert akv._TORCH_DECODE is not None, "libaicomp_kv_torch.so is not built"
+    monkeypatch.setattr(akv, "_route", request.param)
     return request.param

@@ -151,19 +151,24 @@ def test_adapter_batch_one_and_hf_style_views(device, host_route):
     new.disable()
 
 
-@pytest.mark.parametrize("route", ["torch_op", "ctypes"])
+@pytest.mark.parametrize("route", ["fast", "torch_op", "ctypes"])
 def test_manager_mode_decode_is_one_fused_call_and_equals_internal_mode(device, monkeypatch, route):
     """With a manager attached (the engine's ``--use-kv-manager`` mode, kv_cache.py:378-381) a decode
     step takes the same fused append + attention call as internal mode: one library call per layer
-    and token, output and pools bit-identical to the internal-mode operator.  Both host routes to
-    the library: the registered PyTorch operator and the ctypes binding."""
+    and token, output and pools bit-identical to the internal-mode operator.  All three host routes
+    to the library: the CPython function, the registered PyTorch operator and the ctypes binding."""
+    import types
     from aicomp_amd import _lib
-    if route == "ctypes":
-        monkeypatch.setattr(akv, "_TORCH_DECODE", None)
-    else:
+    monkeypatch.setattr(akv, "_route", route)
+    if route == "torch_op":
         real_op = akv._TORCH_DECODE
         assert real_op is not None
         monkeypatch.setattr(akv, "_TORCH_DECODE", lambda *a: (calls.append("torch_op.decode_step"), real_op(*a))[1])
+    elif route == "fast":
+        real_fast = akv._FAST
+        assert real_fast is not None
+        monkeypatch.setattr(akv, "_FAST", types.SimpleNamespace(
+            layer=real_fast.layer, decode_step=lambda *a: (calls.append("fast.decode_step"), real_fast.decode_step(*a))[1]))
     B, hq, g, d, layers = 3, 16, 4, 128, 2
     hkv = hq // g
     mgr = akv.KVCacheManager(num_layers=layers, max_batch_size=4, max_seq_len=128, num_heads=hq, head_dim=d,
@@ -205,7 +210,8 @@ def test_manager_mode_decode_is_one_fused_call_and_equals_internal_mode(device, 
                     setattr(lib, s, real[s])
             assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"n={n} layer {layer}"
             if n == 1:
-                assert calls == (["aicomp_paged_decode_attn_append"] if route == "ctypes" else ["torch_op.decode_step"]), calls
+                assert calls == [{"ctypes": "aicomp_paged_decode_attn_append", "torch_op": "torch_op.decode_step",
+                                  "fast": "fast.decode_step"}[route]], calls
             else:
                 assert calls == ["aicomp_kv_append", "aicomp_paged_prefill_attn"], calls
         assert mgr.get_seq_len() == ext[0].cache_pos == own[0].cache_pos

@@ -117,3 +117,41 @@ def test_registered_ops_reject_bad_arguments_with_runtime_errors(device):
         q = torch.zeros(2, 32, 1, 128, dtype=torch.bfloat16, device=device)
         k = torch.zeros(2, 8, 1, 128, dtype=torch.bfloat16, device=device)
         t.decode_step(q, k, k, layer.k_pool, layer.v_pool, layer.block_table, layer.ctx_rows, 64, 4, 0.1, None)
+
+
+@pytest.mark.parametrize("B,hq,g,d,dtype", [(1, 32, 4, 64, torch.bfloat16), (3, 16, 4, 128, torch.float16), (2, 8, 2, 64, torch.float32)])
+def test_lean_decode_call_equals_the_registered_op(device, B, hq, g, d, dtype):
+    """aicomp_amd._aicomp_fast.decode_step (a layer's static tensors behind a handle, one CPython
+    call per step) against torch.ops.mi355_kv.decode_step: same output bits, same pools, across a
+    block boundary and the point where the call starts to need a merge (640 tokens)."""
+    from aicomp_amd import _aicomp_fast as fast
+    t = _lib.torch_ops()
+    hkv = hq // g
+    a = akv._PagedLayer(B, hkv, d, 1024, dtype, device)
+    b = akv._PagedLayer(B, hkv, d, 1024, dtype, device)
+    gen = torch.Generator().manual_seed(B + d)
+    mk = lambda n, h: torch.randn(B, h, n, d, generator=gen).to(dtype).to(device)
+    k0, v0 = mk(636, hkv), mk(636, hkv)
+    a.append(k0, v0, 0, 1)
+    b.append(k0, v0, 0, 1)
+    handle = fast.layer(a.k_pool, a.v_pool, a.block_table, a.ctx_rows)
+    for pos in range(636, 644):
+        q, k, v = mk(1, hq), mk(1, hkv).repeat_interleave(g, 1), mk(1, hkv).repeat_interleave(g, 1)
+        got = fast.decode_step(handle, q, k, v, pos, g, 1 / math.sqrt(d))
+        want = t.decode_step(q, k, v, b.k_pool, b.v_pool, b.block_table, b.ctx_rows, pos, g, 1 / math.sqrt(d), None)
+        assert got.shape == want.shape and got.dtype == dtype and torch.equal(bits(got), bits(want)), pos
+    assert torch.equal(bits(a.k_pool), bits(b.k_pool)) and torch.equal(bits(a.v_pool), bits(b.v_pool))
+    # a transposed (non-contiguous) query and strided K/V views are taken as they are or copied, as in the op
+    q = mk(1, hq).transpose(1, 3).contiguous().transpose(1, 3)
+    k = mk(1, hkv)
+    got = fast.decode_step(handle, q, k, k, 644, g, 0.1)
+    want = t.decode_step(q, k, k, b.k_pool, b.v_pool, b.block_table, b.ctx_rows, 644, g, 0.1, None)
+    assert torch.equal(bits(got), bits(want))
+    for bad in (lambda: fast.decode_step(handle, q[:, :, :, :8], k, k, 645, g, 0.1),               # head_dim
+                lambda: fast.decode_step(handle, q, mk(1, hkv + 1), mk(1, hkv + 1), 645, g, 0.1),  # K/V heads
+                lambda: fast.decode_step(handle, q.float() if dtype != torch.float32 else q.half(), k, k, 645, g, 0.1),
+                lambda: fast.decode_step(handle, q, k, k, 5000, g, 0.1),                            # beyond ctx_rows
+                lambda: fast.decode_step(handle, q.cpu(), k, k, 645, g, 0.1),
+                lambda: fast.layer(a.k_pool.cpu(), a.v_pool.cpu(), a.block_table.cpu(), a.ctx_rows.cpu())):
+        with pytest.raises(RuntimeError):
+            bad()
