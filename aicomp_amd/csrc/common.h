@@ -201,6 +201,27 @@ struct F16Fmt {
     static constexpr uint32_t SIGN_PAIR = 0x80008000u;
 };
 
+// --------------------------------------- order of query tiles in a prefill grid ---
+// A prefill grid is (head group, sequence, query tile slice), dispatched x fastest: the first
+// num_cus workgroups land one per CU, the next num_cus beside them, the rest as places free up.
+// A query tile of a causal chunk costs as many steps as it has keys, so tile index = cost order.
+// A grid of at most two workgroups per CU is resident all at once, so which two share a CU decides
+// when the kernel ends: its slices are handed out in rounds of num_cus workgroups, the first from
+// the expensive end downwards and the second from the cheap end upwards, so that the two
+// workgroups of a CU are the p-th most expensive and the p-th cheapest tile (a fresh 2048-token
+// prompt is 512 workgroups: expensive first, CU 0 gets tiles 63 and 31 and CU 255 tiles 32 and 0;
+// this way every CU gets 63 steps: 482 -> 382 us for such a float32 prompt).  Larger grids are
+// dispatched as places free up, and there expensive first is the better order (an 8192-token
+// prompt: 470 us against 498 us zig-zag).  Returns the tile of slice z (a bijection of 0 .. Z-1
+// for any Z).
+__device__ __forceinline__ int prefill_tile_of_slice(int z, int Z, int num_cus, int wgs_per_slice) {
+    if (num_cus <= 0 || wgs_per_slice <= 0 || num_cus % wgs_per_slice != 0 || Z * wgs_per_slice > 2 * num_cus)
+        return Z - 1 - z;
+    const int per_round = num_cus / wgs_per_slice;
+    const int k = z / per_round, pos = z - k * per_round;
+    return (k & 1) ? (k >> 1) * per_round + pos : Z - 1 - (k >> 1) * per_round - pos;
+}
+
 // ------------------------------------------------- split-K workspace view ---
 // part_acc [rows][Hq][P][D] float : sum_j 2^(s_j - m) v_j   (not normalised)
 // part_ml  [rows][Hq][P][2] float : m (log2 domain), l = sum_j 2^(s_j - m)

@@ -147,8 +147,10 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     // a CU from the start are then a long item and a short one, and later places are handed out
     // longest first.  An item's rank comes in closed form from the other chunks' lengths (its
     // cost c, then per chunk the number of tiles costing >= c and >= c + 1), so the work is per
-    // chunk, not per item.  Other grids keep the grid order, longest tile of every chunk first.
-    int seq = blockIdx.y, qtile = gridDim.z - 1 - blockIdx.z;
+    // chunk, not per item.  Other grids (a single prompt, many chunks) take their query tile slices in
+    // the order of prefill_tile_of_slice: expensive first, or, when the whole grid is resident at
+    // once, expensive and cheap tiles paired on a CU.
+    int seq = blockIdx.y, qtile = prefill_tile_of_slice(blockIdx.z, gridDim.z, p.num_cus, gridDim.x * gridDim.y);
     const int nseq = gridDim.y, ntile = gridDim.z, items = nseq * ntile;
     bool ranked = false;
     int r_ctx = 0, r_n = 0, r_qb = 0;

@@ -47,6 +47,7 @@ struct PrefillF32Params {
     const int32_t* cu_q_lens;
     int hq, hkv, group, gpack, max_blocks;
     int num_blocks;
+    int num_cus;                        // CUs of the device (0: expensive tiles first)
     float qk_mul;
 };
 
@@ -62,7 +63,7 @@ paged_prefill_mfma_f32_kernel(PrefillF32Params p) {
     constexpr int NL = KT / RPL;                // loads per tile and pool (4 or 2)
     const int hgroup = blockIdx.x;
     const int seq = blockIdx.y;
-    const int qtile = gridDim.z - 1 - blockIdx.z;       // longest query tiles first
+    const int qtile = prefill_tile_of_slice(blockIdx.z, gridDim.z, p.num_cus, gridDim.x * gridDim.y);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -297,6 +298,18 @@ int launch_prefill_mfma_f32(const DecodeArgs& a, int max_q_len) {
     p.num_blocks = (int)a.num_blocks;
     p.gpack = (16 % p.group == 0) ? p.group : 1;
     p.qk_mul = a.scale * LOG2E;
+    // CU count of the first device used (every GPU of a node is the same part); 0 if unknown
+    static std::atomic<int> cached_cus{-1};
+    int num_cus = cached_cus.load(std::memory_order_relaxed);
+    if (num_cus < 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 0)
+            n = 0;
+        num_cus = n;
+        cached_cus.store(n, std::memory_order_relaxed);
+    }
+    p.num_cus = num_cus;
     const int pos_per_wg = WG_ROWS / p.gpack;
     const int qtiles = (max_q_len + pos_per_wg - 1) / pos_per_wg;
     AICOMP_REQUIRE(qtiles <= 65535, AICOMP_KV_EINVAL, "paged_prefill_attn: grid too large");

@@ -556,6 +556,7 @@ def prefill_shapes_bench(dev, reps=20):
     hq, hkv = 32, 8
     out = []
     for nseq, n, prior, d, kvt, qt in ((1, 8192, 0, 128, torch.bfloat16, torch.bfloat16),
+                                       (1, 2048, 0, 128, torch.bfloat16, torch.bfloat16),
                                        (4, 4096, 0, 128, torch.bfloat16, torch.bfloat16),
                                        (16, 512, 2048, 128, torch.bfloat16, torch.bfloat16),
                                        (16, 512, 2048, 128, torch.float8_e4m3fn, torch.bfloat16),
