@@ -168,6 +168,24 @@ def test_prefill_fp32_matrix_kernel_ignores_everything_beyond_the_context(device
     assert np.abs(to_f64(got) - oracle(c)).max() <= 1e-5
 
 
+@pytest.mark.parametrize("n,dtype", [(1024, torch.bfloat16), (1500, torch.bfloat16), (2048, torch.bfloat16),
+                                     (1500, torch.float32), (700, torch.float16)])
+def test_single_prompt_whose_grid_is_resident_at_once(device, n, dtype):
+    """A fresh prompt of at most two workgroups per CU takes its query tiles in paired order (an
+    expensive and a cheap tile per CU): one round, two full rounds, and a second round that is only
+    partly filled.  Every row must still be computed exactly once (the output starts as NaN) and
+    match the float64 oracle."""
+    c = build_case(device, priors=[0], news=[n], hq=32, hkv=8, d=128, dtype=dtype, seed=n, poison=False)
+    got = run(c)
+    assert torch.isfinite(got.float()).all()
+    want = orc.paged_prefill_attn(raw(c["q"]), raw(c["k_pool"]), raw(c["v_pool"]), c["table"].cpu().numpy(), [n], [0, n],
+                                  c["scale"], NAME[dtype], NAME[dtype], gather=orc.gather_context_fast)
+    if dtype == torch.float32:
+        assert np.abs(to_f64(got) - want).max() <= 1e-5
+    else:
+        assert_close_attn(to_f64(got), want, BF16_ATOL, BF16_RTOL, f"{n}-token prompt, {dtype}")
+
+
 def test_prefill_fp32_long_prompt_all_rows(device):
     """A fresh 2048-token float32 prompt at the Llama-3 head shape (the bench's float32 shape): every
     row within 1e-5 of the float64 oracle, and equal to torch's own is_causal=True float32 SDPA on
