@@ -241,7 +241,9 @@ paged_prefill_mfma_kernel(PrefillParams p) {
         qabs[c] = row_valid[c] ? prior + qpos[c] : ctx - 1;    // padded rows: computed, never stored
     }
     // last key any row of this wave / workgroup may see (exclusive)
-    const int wave_kv_end = min(ctx, prior + q0 + (WROWS * w + WROWS - 1) / p.gpack + 1);
+    // (a wave whose rows all lie beyond the chunk's end has nothing to compute: it only takes part in
+    // the tile loads and barriers)
+    const int wave_kv_end = q0 + (WROWS * w) / p.gpack >= n ? 0 : min(ctx, prior + q0 + (WROWS * w + WROWS - 1) / p.gpack + 1);
     const int wave_kv_min = prior + q0 + (WROWS * w) / p.gpack;    // smallest qabs in the wave (if valid)
     const int kv_end = min(ctx, prior + q0 + pos_per_wg);
     const int ntiles = (kv_end + TT - 1) / TT;

@@ -100,7 +100,9 @@ paged_prefill_mfma_f32_kernel(PrefillF32Params p) {
         row_valid[c] = qpos[c] < n;
         qabs[c] = row_valid[c] ? prior + qpos[c] : ctx - 1;     // padded rows: computed, never stored
     }
-    const int wave_kv_end = min(ctx, prior + q0 + (16 * R * w + 16 * R - 1) / p.gpack + 1);
+    // (a wave whose rows all lie beyond the chunk's end has nothing to compute: it only takes part in
+    // the tile loads and barriers)
+    const int wave_kv_end = q0 + (16 * R * w) / p.gpack >= n ? 0 : min(ctx, prior + q0 + (16 * R * w + 16 * R - 1) / p.gpack + 1);
     const int wave_kv_min = prior + q0 + (16 * R * w) / p.gpack;
     const int kv_end = min(ctx, prior + q0 + pos_per_wg);
     const int ntiles = (kv_end + KT - 1) / KT;
