@@ -23,6 +23,8 @@ SYMBOLS = (
     "aicomp_paged_decode_workspace_bytes",
     "aicomp_paged_decode_partition_size",
     "aicomp_paged_prefill_attn",
+    "aicomp_paged_prefill_attn_items",
+    "aicomp_paged_prefill_tile_positions",
     "aicomp_rope_kv_append",
     "aicomp_sample_tokens",
 )
@@ -67,6 +69,12 @@ def _declare(lib: C.CDLL) -> None:
     lib.aicomp_paged_prefill_attn.argtypes = [vp, vp, vp, vp, vp, i64, vp, vp, i32, i64, i32,
                                               i32, i32, i32, i32, i32, i64, f32, i32, i32,
                                               vp, vp, vp]
+    lib.aicomp_paged_prefill_attn_items.restype = i32
+    lib.aicomp_paged_prefill_attn_items.argtypes = [vp, vp, vp, vp, vp, i64, vp, vp, i32, i64, i32,
+                                                    i32, i32, i32, i32, i32, i64, f32, i32, i32,
+                                                    vp, vp, vp, i32, vp]
+    lib.aicomp_paged_prefill_tile_positions.restype = i32
+    lib.aicomp_paged_prefill_tile_positions.argtypes = [i32] * 7
     lib.aicomp_rope_kv_append.restype = i32
     lib.aicomp_rope_kv_append.argtypes = [vp, vp, i64, i64, i64, i64, vp, vp, i64, i64, vp, vp, i64, i64, vp,
                                           vp, vp, vp, i64, i32, i32, i32, i32, i64, i32, i32, vp, vp, vp]

@@ -184,6 +184,32 @@ class StepPlan:
     host_cu_q_lens: np.ndarray = None
     host_slot_mapping: np.ndarray = None
     host_positions: np.ndarray = None
+    # order of the prompt chunks' query tiles per (tile size, head groups): one list serves every layer of the step
+    _prefill_items: dict = None
+
+    def prefill_items(self, query: torch.Tensor, k_pool: torch.Tensor) -> Optional[torch.Tensor]:
+        """The (sequence, query tile) pairs of this step's prompt chunks, most expensive first, as the
+        device tensor ``ops.paged_prefill_attn(items=...)`` takes; ``None`` when the step has fewer
+        than two chunks (the kernel's own order is as good) or the kernel at hand takes no list.
+        Built once per step from the host copies of the lengths and reused by every layer."""
+        from . import ops
+        npre = self.num_prefill_seqs
+        if npre < 2:
+            return None
+        hq, hkv, d, bs = query.shape[1], k_pool.shape[1], k_pool.shape[3], k_pool.shape[2]
+        tile = ops.prefill_tile_positions(hq, hkv, d, bs, query.dtype, k_pool.dtype, self.max_q_len)
+        if tile <= 0:
+            return None
+        group = hq // hkv
+        hgroups = hq // (group if 16 % group == 0 else 1)
+        key = (tile, hgroups, query.device)
+        if self._prefill_items is None:
+            self._prefill_items = {}
+        if key not in self._prefill_items:
+            cus = torch.cuda.get_device_properties(query.device).multi_processor_count if query.is_cuda else 0
+            items = ops.prefill_items(self.host_context_lens[:npre], self.new_lens[:npre], tile, hgroups, cus)
+            self._prefill_items[key] = torch.from_numpy(items).to(query.device, non_blocking=True)
+        return self._prefill_items[key]
 
     @property
     def num_seqs(self) -> int:
@@ -548,7 +574,8 @@ def paged_attention_step(plan: StepPlan, out: torch.Tensor, query: torch.Tensor,
         ops.kv_append(key[:t_pre], value[:t_pre], k_pool, v_pool, plan.slot_mapping[:t_pre], k_scale, v_scale)
         ops.paged_prefill_attn(out[:t_pre], query[:t_pre], k_pool, v_pool, plan.block_table[:npre],
                                plan.context_lens[:npre], plan.cu_q_lens[:npre + 1], scale,
-                               max_q_len=plan.max_q_len, k_scale=k_scale, v_scale=v_scale)
+                               max_q_len=plan.max_q_len, k_scale=k_scale, v_scale=v_scale,
+                               items=plan.prefill_items(query, k_pool))
     if S > npre:
         ops.paged_decode_attn(out[t_pre:], query[t_pre:], k_pool, v_pool, plan.block_table[npre:],
                               plan.context_lens[npre:], scale, k_scale, v_scale,

@@ -31,6 +31,8 @@ int launch_kv_append(const void* key, const void* value, int64_t token_stride, i
 
 bool prefill_mfma_supported(const DecodeArgs& a, int max_q_len);
 int launch_prefill_mfma(const DecodeArgs& a, int max_q_len);
+int prefill_mfma_tile_positions(int hq, int hkv, int max_q_len);
+int prefill_mfma_f32_tile_positions(int hq, int hkv);
 bool prefill_mfma_f32_supported(const DecodeArgs& a, int max_q_len);
 int launch_prefill_mfma_f32(const DecodeArgs& a, int max_q_len);
 bool prefill_tiled_supported(const DecodeArgs& a, int max_q_len);
@@ -410,13 +412,14 @@ int aicomp_paged_decode_attn_append_static(void* out, const void* query, const v
                        k_scale, v_scale, partition_size, ws, need, stream, who);
 }
 
-int aicomp_paged_prefill_attn(void* out, const void* query, const void* k_pool, const void* v_pool,
-                              const int32_t* block_table, int64_t block_table_stride,
-                              const int32_t* context_lens, const int32_t* cu_q_lens, int num_seqs,
-                              int64_t total_q, int max_q_len, int num_q_heads, int num_kv_heads,
-                              int head_dim, int block_size, int max_blocks_per_seq,
-                              int64_t num_blocks, float scale, int q_dtype, int kv_dtype,
-                              const float* k_scale, const float* v_scale, void* stream) {
+static int prefill_impl(void* out, const void* query, const void* k_pool, const void* v_pool,
+                        const int32_t* block_table, int64_t block_table_stride,
+                        const int32_t* context_lens, const int32_t* cu_q_lens, int num_seqs,
+                        int64_t total_q, int max_q_len, int num_q_heads, int num_kv_heads,
+                        int head_dim, int block_size, int max_blocks_per_seq,
+                        int64_t num_blocks, float scale, int q_dtype, int kv_dtype,
+                        const float* k_scale, const float* v_scale, const int32_t* items, int num_items,
+                        void* stream) {
     AICOMP_REQUIRE(num_seqs >= 0 && total_q >= 0, AICOMP_KV_EINVAL,
                    "paged_prefill_attn: negative sizes");
     if (num_seqs == 0 || total_q == 0) return AICOMP_KV_OK;
@@ -431,6 +434,8 @@ int aicomp_paged_prefill_attn(void* out, const void* query, const void* k_pool, 
     AICOMP_REQUIRE(max_blocks_per_seq > 0 && block_table_stride >= max_blocks_per_seq,
                    AICOMP_KV_EINVAL, "paged_prefill_attn: block table stride %lld < width %d",
                    (long long)block_table_stride, max_blocks_per_seq);
+    AICOMP_REQUIRE(items == nullptr || num_items > 0, AICOMP_KV_EINVAL,
+                   "paged_prefill_attn: an item list needs at least one item");
     DecodeArgs a;
     memset(&a, 0, sizeof(a));
     a.out = out; a.query = query; a.k_pool = k_pool; a.v_pool = v_pool;
@@ -443,6 +448,9 @@ int aicomp_paged_prefill_attn(void* out, const void* query, const void* k_pool, 
     a.k_scale = kv_dtype == AICOMP_KV_FP8_E4M3 ? k_scale : nullptr;
     a.v_scale = kv_dtype == AICOMP_KV_FP8_E4M3 ? v_scale : nullptr;
     a.stream = (hipStream_t)stream;
+    // an item list is taken by the two matrix-instruction kernels (and only while its length fits a
+    // grid dimension); the other kernels walk the whole grid, which covers the same tiles
+    if (items != nullptr && num_items <= 65535) { a.items = items; a.num_items = num_items; }
     if (prefill_mfma_supported(a, max_q_len)) return launch_prefill_mfma(a, max_q_len);
     // float32 models at head_dim 64 / 128: the float32 matrix instruction
     if (prefill_mfma_f32_supported(a, max_q_len)) return launch_prefill_mfma_f32(a, max_q_len);
@@ -455,6 +463,47 @@ int aicomp_paged_prefill_attn(void* out, const void* query, const void* k_pool, 
                              block_size * block_size);
     a.num_parts = 1;
     return launch_decode_generic(a);
+}
+
+int aicomp_paged_prefill_attn(void* out, const void* query, const void* k_pool, const void* v_pool,
+                              const int32_t* block_table, int64_t block_table_stride,
+                              const int32_t* context_lens, const int32_t* cu_q_lens, int num_seqs,
+                              int64_t total_q, int max_q_len, int num_q_heads, int num_kv_heads,
+                              int head_dim, int block_size, int max_blocks_per_seq,
+                              int64_t num_blocks, float scale, int q_dtype, int kv_dtype,
+                              const float* k_scale, const float* v_scale, void* stream) {
+    return prefill_impl(out, query, k_pool, v_pool, block_table, block_table_stride, context_lens, cu_q_lens,
+                        num_seqs, total_q, max_q_len, num_q_heads, num_kv_heads, head_dim, block_size,
+                        max_blocks_per_seq, num_blocks, scale, q_dtype, kv_dtype, k_scale, v_scale, nullptr, 0,
+                        stream);
+}
+
+int aicomp_paged_prefill_attn_items(void* out, const void* query, const void* k_pool, const void* v_pool,
+                                    const int32_t* block_table, int64_t block_table_stride,
+                                    const int32_t* context_lens, const int32_t* cu_q_lens, int num_seqs,
+                                    int64_t total_q, int max_q_len, int num_q_heads, int num_kv_heads,
+                                    int head_dim, int block_size, int max_blocks_per_seq,
+                                    int64_t num_blocks, float scale, int q_dtype, int kv_dtype,
+                                    const float* k_scale, const float* v_scale, const int32_t* items,
+                                    int num_items, void* stream) {
+    AICOMP_REQUIRE(num_items >= 0 && (items != nullptr || num_items == 0), AICOMP_KV_EINVAL,
+                   "paged_prefill_attn_items: %d items without a list", num_items);
+    return prefill_impl(out, query, k_pool, v_pool, block_table, block_table_stride, context_lens, cu_q_lens,
+                        num_seqs, total_q, max_q_len, num_q_heads, num_kv_heads, head_dim, block_size,
+                        max_blocks_per_seq, num_blocks, scale, q_dtype, kv_dtype, k_scale, v_scale,
+                        num_items > 0 ? items : nullptr, num_items, stream);
+}
+
+int aicomp_paged_prefill_tile_positions(int num_q_heads, int num_kv_heads, int head_dim, int block_size,
+                                        int q_dtype, int kv_dtype, int max_q_len) {
+    if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads || max_q_len <= 0 || block_size != 16 ||
+        (head_dim != 64 && head_dim != 128))
+        return 0;
+    if (is_16bit_float(q_dtype) && (kv_dtype == q_dtype || kv_dtype == AICOMP_KV_FP8_E4M3))
+        return prefill_mfma_tile_positions(num_q_heads, num_kv_heads, max_q_len);
+    if (q_dtype == AICOMP_KV_F32 && kv_dtype == AICOMP_KV_F32)
+        return prefill_mfma_f32_tile_positions(num_q_heads, num_kv_heads);
+    return 0;
 }
 
 }  // extern "C"

@@ -269,6 +269,10 @@ struct DecodeArgs {
     const void* new_key;
     const void* new_value;
     int64_t new_token_stride, new_head_stride;
+    // prefill only (NULL = none): (sequence, query tile) pairs, one workgroup row each, in the order
+    // the workgroups are to take them
+    const int32_t* items;
+    int num_items;
 };
 
 int launch_decode_generic(const DecodeArgs& a);

@@ -66,6 +66,8 @@ struct PrefillParams {
     float qk_mul;
     const float* k_scale;
     const float* v_scale;
+    const int32_t* items;              // (sequence, query tile) pairs; grid.y numbers them (NULL: none)
+    int num_seqs;
 };
 
 // max over lanes l and l^16 (l^32): gfx950's lane-swap instructions, no LDS round trip.
@@ -154,7 +156,13 @@ paged_prefill_mfma_kernel(PrefillParams p) {
     const int nseq = gridDim.y, ntile = gridDim.z, items = nseq * ntile;
     bool ranked = false;
     int r_ctx = 0, r_n = 0, r_qb = 0;
-    if (p.num_cus > 0 && nseq > 1 && nseq <= 16 && items <= 256) {     // workgroup-uniform
+    if (p.items != nullptr) {
+        // The caller ranked the items itself (it knows the lengths on the host): workgroup row y
+        // takes pair y.  A pair that names no sequence is skipped; a tile beyond its chunk exits below.
+        seq = p.items[2 * blockIdx.y];
+        qtile = p.items[2 * blockIdx.y + 1];
+        if (seq < 0 || seq >= p.num_seqs || qtile < 0) return;
+    } else if (p.num_cus > 0 && nseq > 1 && nseq <= 16 && items <= 256) {     // workgroup-uniform
         int* scratch = (int*)(DMA ? dma_k0 : lds);                     // the tile buffers are still unused
         if (tid < nseq) {
             const int qb_t = p.cu_q_lens[tid];
@@ -692,6 +700,14 @@ bool prefill_mfma_supported(const DecodeArgs& a, int max_q_len) {
            ((uintptr_t)a.v_pool % 16 == 0);
 }
 
+// positions of one query tile (one workgroup row) for these shapes: what an item list is cut into
+int prefill_mfma_tile_positions(int hq, int hkv, int max_q_len) {
+    const int group = hq / hkv;
+    const int gpack = (16 % group == 0) ? group : 1;
+    const int R = (int64_t)max_q_len * gpack >= 2 * ROWS ? 2 : 1;
+    return ROWS * R / gpack;
+}
+
 int launch_prefill_mfma(const DecodeArgs& a, int max_q_len) {
     PrefillParams p;
     p.out = a.out; p.query = a.query; p.k_pool = a.k_pool; p.v_pool = a.v_pool;
@@ -716,12 +732,14 @@ int launch_prefill_mfma(const DecodeArgs& a, int max_q_len) {
     p.num_cus = num_cus;
     p.qk_mul = a.scale * LOG2E;
     p.k_scale = a.k_scale; p.v_scale = a.v_scale;
+    p.items = a.items; p.num_seqs = a.num_seqs;
     // two column groups per wave (128 rows per workgroup) once a chunk has that many rows
     const int R = (int64_t)max_q_len * p.gpack >= 2 * ROWS ? 2 : 1;
     const int pos_per_wg = ROWS * R / p.gpack;
     const int qtiles = (max_q_len + pos_per_wg - 1) / pos_per_wg;
     AICOMP_REQUIRE(qtiles <= 65535, AICOMP_KV_EINVAL, "paged_prefill_attn: grid too large");
     dim3 grid((unsigned)(a.hq / p.gpack), (unsigned)a.num_seqs, (unsigned)qtiles);
+    if (a.items != nullptr) grid = dim3((unsigned)(a.hq / p.gpack), (unsigned)a.num_items, 1);
     // double-buffered K and V tiles of 32 (R = 1) or 64 rows of 2*D + 16 bytes
     const size_t lds_bytes = (size_t)4 * (R == 1 ? 32 : 64) * (2 * a.d + 16);
     const bool fp8 = a.kv_dtype == AICOMP_KV_FP8_E4M3;

@@ -49,6 +49,8 @@ struct PrefillF32Params {
     int num_blocks;
     int num_cus;                        // CUs of the device (0: expensive tiles first)
     float qk_mul;
+    const int32_t* items;               // (sequence, query tile) pairs; grid.y numbers them (NULL: none)
+    int num_seqs;
 };
 
 template <int DH>
@@ -62,8 +64,13 @@ paged_prefill_mfma_f32_kernel(PrefillF32Params p) {
     constexpr int RPL = 256 / CPR;              // rows one load of the workgroup covers (8 or 16)
     constexpr int NL = KT / RPL;                // loads per tile and pool (4 or 2)
     const int hgroup = blockIdx.x;
-    const int seq = blockIdx.y;
-    const int qtile = prefill_tile_of_slice(blockIdx.z, gridDim.z, p.num_cus, gridDim.x * gridDim.y);
+    int seq = blockIdx.y;
+    int qtile = prefill_tile_of_slice(blockIdx.z, gridDim.z, p.num_cus, gridDim.x * gridDim.y);
+    if (p.items != nullptr) {           // the caller's own order: workgroup row y takes pair y
+        seq = p.items[2 * blockIdx.y];
+        qtile = p.items[2 * blockIdx.y + 1];
+        if (seq < 0 || seq >= p.num_seqs || qtile < 0) return;
+    }
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -290,6 +297,11 @@ bool prefill_mfma_f32_supported(const DecodeArgs& a, int max_q_len) {
            ((uintptr_t)a.out % 16 == 0) && ((uintptr_t)a.k_pool % 16 == 0) && ((uintptr_t)a.v_pool % 16 == 0);
 }
 
+int prefill_mfma_f32_tile_positions(int hq, int hkv) {
+    const int group = hq / hkv;
+    return WG_ROWS / ((16 % group == 0) ? group : 1);
+}
+
 int launch_prefill_mfma_f32(const DecodeArgs& a, int max_q_len) {
     PrefillF32Params p;
     p.out = (float*)a.out; p.query = (const float*)a.query;
@@ -312,10 +324,12 @@ int launch_prefill_mfma_f32(const DecodeArgs& a, int max_q_len) {
         cached_cus.store(n, std::memory_order_relaxed);
     }
     p.num_cus = num_cus;
+    p.items = a.items; p.num_seqs = a.num_seqs;
     const int pos_per_wg = WG_ROWS / p.gpack;
     const int qtiles = (max_q_len + pos_per_wg - 1) / pos_per_wg;
     AICOMP_REQUIRE(qtiles <= 65535, AICOMP_KV_EINVAL, "paged_prefill_attn: grid too large");
     dim3 grid((unsigned)(a.hq / p.gpack), (unsigned)a.num_seqs, (unsigned)qtiles);
+    if (a.items != nullptr) grid = dim3((unsigned)(a.hq / p.gpack), (unsigned)a.num_items, 1);
     const hipError_t e = a.d == 64 ? launch_f32_variant<64>(p, grid, a.stream) : launch_f32_variant<128>(p, grid, a.stream);
     AICOMP_REQUIRE(e == hipSuccess, AICOMP_KV_EHIP, "paged_prefill_attn: %s", hipGetErrorString(e));
     AICOMP_HIP_LAUNCH_CHECK();

@@ -200,7 +200,7 @@ void paged_decode_attn_append(at::Tensor& out, const at::Tensor& query, const at
 void paged_prefill_attn(at::Tensor& out, const at::Tensor& query, const at::Tensor& k_pool, const at::Tensor& v_pool,
                         const at::Tensor& block_table, const at::Tensor& context_lens, const at::Tensor& cu_q_lens,
                         double scale, int64_t max_q_len, const c10::optional<at::Tensor>& k_scale,
-                        const c10::optional<at::Tensor>& v_scale) {
+                        const c10::optional<at::Tensor>& v_scale, const c10::optional<at::Tensor>& items) {
     const Pools p = check_pools(k_pool, v_pool);
     TORCH_CHECK(query.dim() == 3 && out.sizes() == query.sizes() && out.scalar_type() == query.scalar_type(),
                 "out/query must both be [T, Hq, D]; got ", out.sizes(), " and ", query.sizes());
@@ -214,12 +214,21 @@ void paged_prefill_attn(at::Tensor& out, const at::Tensor& query, const at::Tens
     TORCH_CHECK(max_q_len > 0 || query.size(0) == 0, "max_q_len must be the host-side bound on the chunk lengths");
     const float *ks, *vs;
     scales(k_pool, k_scale, v_scale, p.hkv, ks, vs);
-    check_rc(aicomp_paged_prefill_attn(out.data_ptr(), query.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(),
-                                       block_table.data_ptr<int32_t>(), block_table.stride(0),
-                                       context_lens.data_ptr<int32_t>(), cu_q_lens.data_ptr<int32_t>(), (int)S,
-                                       query.size(0), (int)max_q_len, (int)query.size(1), p.hkv, p.d, p.bs,
-                                       (int)block_table.size(1), p.nb, (float)scale, dtype_code(query, "query"),
-                                       dtype_code(k_pool, "pool"), ks, vs, stream_of(query)));
+    const int32_t* item_ptr = nullptr;
+    int num_items = 0;
+    if (items.has_value() && items->numel() > 0) {
+        TORCH_CHECK(items->scalar_type() == at::kInt && items->dim() == 2 && items->size(1) == 2 && items->is_contiguous() &&
+                    items->device() == query.device(),
+                    "items must be a contiguous int32 [n, 2] tensor of (sequence, query tile) pairs on ", query.device());
+        item_ptr = items->data_ptr<int32_t>();
+        num_items = (int)items->size(0);
+    }
+    check_rc(aicomp_paged_prefill_attn_items(out.data_ptr(), query.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(),
+                                             block_table.data_ptr<int32_t>(), block_table.stride(0),
+                                             context_lens.data_ptr<int32_t>(), cu_q_lens.data_ptr<int32_t>(), (int)S,
+                                             query.size(0), (int)max_q_len, (int)query.size(1), p.hkv, p.d, p.bs,
+                                             (int)block_table.size(1), p.nb, (float)scale, dtype_code(query, "query"),
+                                             dtype_code(k_pool, "pool"), ks, vs, item_ptr, num_items, stream_of(query)));
 }
 
 at::Tensor decode_step(const at::Tensor& query_in, const at::Tensor& key, const at::Tensor& value, at::Tensor& k_pool,
@@ -284,7 +293,7 @@ TORCH_LIBRARY(mi355_kv, m) {
           "Tensor? v_scale=None, int partition_size=0, Tensor? workspace=None) -> ()");
     m.def("paged_prefill_attn(Tensor(a!) out, Tensor query, Tensor k_pool, Tensor v_pool, Tensor block_table, "
           "Tensor context_lens, Tensor cu_q_lens, float scale, int max_q_len, Tensor? k_scale=None, "
-          "Tensor? v_scale=None) -> ()");
+          "Tensor? v_scale=None, Tensor? items=None) -> ()");
     m.def("decode_step(Tensor query, Tensor key, Tensor value, Tensor(a!) k_pool, Tensor(b!) v_pool, Tensor block_table, "
           "Tensor ctx_rows, int position, int group, float scale, Tensor? workspace=None) -> Tensor");
 }

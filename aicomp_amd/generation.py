@@ -82,7 +82,7 @@ class PagedAttentionBackend:
         if npre:
             ops.paged_prefill_attn(out[:t_pre], q[:t_pre], kp, vp, plan.block_table[:npre], plan.context_lens[:npre],
                                    plan.cu_q_lens[:npre + 1], self.scale, max_q_len=plan.max_q_len,
-                                   k_scale=ks, v_scale=vs)
+                                   k_scale=ks, v_scale=vs, items=plan.prefill_items(q, kp))
         if S > npre:
             ops.paged_decode_attn(out[t_pre:], q[t_pre:], kp, vp, plan.block_table[npre:], plan.context_lens[npre:],
                                   self.scale, ks, vs)

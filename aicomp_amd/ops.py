@@ -333,18 +333,61 @@ class PreparedDecode:
         return out
 
 
+def prefill_tile_positions(num_q_heads: int, num_kv_heads: int, head_dim: int, block_size: int,
+                           q_dtype: torch.dtype, kv_dtype: torch.dtype, max_q_len: int) -> int:
+    """Positions per query tile (one workgroup row) of the kernel a prefill call with these shapes
+    runs on; 0 when that kernel takes no item list."""
+    return _lib.load().aicomp_paged_prefill_tile_positions(num_q_heads, num_kv_heads, head_dim, block_size,
+                                                           _DT[q_dtype], _DT[kv_dtype], int(max_q_len))
+
+
+def prefill_items(context_lens, new_lens, tile_positions: int, num_head_groups: int = 1,
+                  num_cus: int = 0):
+    """The order in which a prefill launch should take its (sequence, query tile) pairs, from the
+    lengths a step planner holds on the host: an ``int32 [n, 2]`` numpy array for
+    ``paged_prefill_attn(items=...)``, every tile that has rows exactly once.
+
+    A tile costs as many steps as its last row has keys (prior context + positions up to the
+    tile's end), and chunks of different priors and lengths differ several-fold, so the list is
+    sorted by that, most expensive first: places that free up go to the longest tiles left.
+    When the whole launch is resident at once (at most two workgroups per CU;
+    ``num_head_groups`` workgroups per item) the second round is handed out from the cheap end
+    instead, so that the two workgroups sharing a CU are an expensive and a cheap tile.
+    """
+    import numpy as np
+    ctx = np.asarray(context_lens, dtype=np.int64)
+    new = np.asarray(new_lens, dtype=np.int64)
+    if tile_positions <= 0 or ctx.shape != new.shape:
+        raise ValueError("prefill_items: tile_positions must be positive and the two length vectors alike")
+    # (a chunk longer than its context, an inconsistent plan, keeps its tiles: the kernel defines its rows as zero)
+    tiles = np.where(new > 0, -(-new // tile_positions), 0)
+    seq = np.repeat(np.arange(ctx.size), tiles)
+    first = np.cumsum(tiles) - tiles
+    q = np.arange(seq.size) - np.repeat(first, tiles)
+    keys = np.minimum(ctx[seq], ctx[seq] - new[seq] + (q + 1) * tile_positions)
+    order = np.argsort(-keys, kind="stable")
+    n = order.size
+    per_round = num_cus // num_head_groups if num_cus > 0 and num_head_groups > 0 and num_cus % num_head_groups == 0 else 0
+    if per_round and per_round < n <= 2 * per_round:
+        # round 0 takes the per_round most expensive tiles in falling order, round 1 the rest in rising order
+        order = np.concatenate([order[:per_round], order[per_round:][::-1]])
+    return np.stack([seq[order], q[order]], axis=1).astype(np.int32)
+
+
 def paged_prefill_attn(out: torch.Tensor, query: torch.Tensor, k_pool: torch.Tensor,
                        v_pool: torch.Tensor, block_table: torch.Tensor,
                        context_lens: torch.Tensor, cu_q_lens: torch.Tensor, scale: float,
                        max_q_len: Optional[int] = None,
                        k_scale: Optional[torch.Tensor] = None,
-                       v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+                       v_scale: Optional[torch.Tensor] = None,
+                       items: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention of concatenated chunks ``query [T, Hq, D]`` over the pool.
 
     Chunk s owns rows ``cu_q_lens[s]:cu_q_lens[s+1]``; its context of
     ``context_lens[s]`` tokens (chunk included) must already be in the pool.
     ``max_q_len`` is the host-side bound on the chunk lengths; when omitted it
-    is read back from ``cu_q_lens`` (a device synchronisation).
+    is read back from ``cu_q_lens`` (a device synchronisation).  ``items`` (``int32 [n, 2]`` on
+    the device, see ``prefill_items``) gives the order of the (sequence, query tile) pairs.
     """
     lib = _lib.load()
     nb, hkv, bs, d = _check_pools(k_pool, v_pool)
@@ -367,6 +410,19 @@ def paged_prefill_attn(out: torch.Tensor, query: torch.Tensor, k_pool: torch.Ten
     if max_q_len is None:
         cu = cu_q_lens.cpu()
         max_q_len = int((cu[1:] - cu[:-1]).max()) if S else 0
+    if items is not None and items.numel():
+        _req(items.dtype == torch.int32 and items.dim() == 2 and items.shape[1] == 2 and items.is_contiguous(),
+             "items must be a contiguous int32 [n, 2] tensor of (sequence, query tile) pairs")
+        _dev(items, query, "items")
+        rc = lib.aicomp_paged_prefill_attn_items(out.data_ptr(), query.data_ptr(), k_pool.data_ptr(),
+                                                 v_pool.data_ptr(), block_table.data_ptr(),
+                                                 block_table.stride(0), context_lens.data_ptr(),
+                                                 cu_q_lens.data_ptr(), S, T, int(max_q_len), hq, hkv, d, bs,
+                                                 block_table.shape[1], nb, float(scale),
+                                                 _dt(query, "query"), _dt(k_pool, "pool"), _ptr(ks), _ptr(vs),
+                                                 items.data_ptr(), items.shape[0], _stream(query))
+        _lib.check(rc, lib)
+        return out
     rc = lib.aicomp_paged_prefill_attn(out.data_ptr(), query.data_ptr(), k_pool.data_ptr(),
                                        v_pool.data_ptr(), block_table.data_ptr(),
                                        block_table.stride(0), context_lens.data_ptr(),

@@ -612,6 +612,81 @@ def prefill_shapes_bench(dev, reps=20):
     return out
 
 
+def prefill_ragged_bench(dev, reps=40):
+    """Ragged chunk batches (a serving step's shape: many chunks of unlike lengths over unlike
+    contexts), once in the order the kernel finds for itself (launch grid, or its own ranking when
+    the batch has at most 16 chunks) and once with the (sequence, query tile) pairs ranked by the
+    caller, ops.prefill_items: the way block_manager.paged_attention_step and generate() call it.
+    The list's upload is outside the timed loop (a planner builds it once per step, with the other
+    step tensors); bf16, 32/8 heads, head_dim 128, block 16; same settle protocol as above."""
+    import itertools
+    import math
+    import random
+    import torch
+    from aicomp_amd import ops
+    hq, hkv, d, bs = 32, 8, 128, 16
+    rnd = random.Random(0)
+    cases = (("32 chunks of 8..512 tokens, priors 0..2048", [rnd.randint(0, 2048) for _ in range(32)],
+              [512, 384, 256, 128, 64, 32, 16, 8] * 4),
+             ("64 chunks of 64 tokens, priors 0..4096", [rnd.randint(0, 4096) for _ in range(64)], [64] * 64),
+             ("4 chunks of 512 + 20 of 48 tokens, priors 0..3000", [rnd.randint(0, 3000) for _ in range(24)],
+              [512] * 4 + [48] * 20))
+    ncu = torch.cuda.get_device_properties(0).multi_processor_count
+    rows = []
+    for name, priors, news in cases:
+        ctx = [p + n for p, n in zip(priors, news)]
+        need = [math.ceil(c / bs) for c in ctx]
+        nb = sum(need) + 1
+        g = torch.Generator().manual_seed(1)
+        perm = torch.randperm(nb - 1, generator=g).to(torch.int32)
+        table = torch.zeros(len(ctx), max(need), dtype=torch.int32)
+        at = 0
+        for s, k_ in enumerate(need):
+            table[s, :k_] = perm[at:at + k_]
+            at += k_
+        table = table.to(dev)
+        k = (torch.randn(nb, hkv, bs, d, device=dev) * 0.5).bfloat16()
+        v = (torch.randn(nb, hkv, bs, d, device=dev) * 0.5).bfloat16()
+        q = torch.randn(sum(news), hq, d, device=dev).bfloat16()
+        o = torch.empty_like(q)
+        cl = torch.tensor(ctx, dtype=torch.int32, device=dev)
+        cu = torch.tensor([0] + list(itertools.accumulate(news)), dtype=torch.int32, device=dev)
+        tile = ops.prefill_tile_positions(hq, hkv, d, bs, q.dtype, k.dtype, max(news))
+        ops.prefill_items(ctx, news, tile, num_head_groups=hkv, num_cus=ncu)        # numpy's first call
+        t0 = time.perf_counter()
+        host_items = ops.prefill_items(ctx, news, tile, num_head_groups=hkv, num_cus=ncu)
+        rank_us = (time.perf_counter() - t0) * 1e6
+        items = torch.from_numpy(host_items).to(dev)
+        us = {}
+        for label, it in (("grid_order", None), ("item_list", items)):
+            call = lambda: ops.paged_prefill_attn(o, q, k, v, table, cl, cu, 1 / math.sqrt(d), max_q_len=max(news),
+                                                  items=it)
+            call()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            while time.perf_counter() - t0 < 0.03:
+                for _ in range(4):
+                    call()
+                torch.cuda.synchronize()
+            e0, e1 = _events(2)
+            e0.record()
+            for _ in range(reps):
+                call()
+            e1.record()
+            torch.cuda.synchronize()
+            us[label] = e0.elapsed_time(e1) / reps * 1e3
+        flops = sum(4 * hq * d * (n * p + n * (n + 1) / 2) for p, n in zip(priors, news))
+        rows.append({"batch": name, "new_tokens": sum(news), "items": int(host_items.shape[0]),
+                     "grid_places": len(news) * math.ceil(max(news) / tile), "tile_positions": tile,
+                     "grid_order_us": round(us["grid_order"], 1), "item_list_us": round(us["item_list"], 1),
+                     "speedup": round(us["grid_order"] / us["item_list"], 2),
+                     "item_list_TFLOPs": round(flops / us["item_list"] / 1e6, 1),
+                     "host_ranking_us": round(rank_us, 1)})
+        del k, v, q, o
+        torch.cuda.empty_cache()
+    return rows
+
+
 def device_info():
     import torch
     p = torch.cuda.get_device_properties(0)
@@ -896,6 +971,7 @@ def main():
         "operator_host_cost": host_cost_bench(dev),
         "mixed_step_streams": mixed_step_bench(dev),
         "prefill_other_shapes": prefill_shapes_bench(dev),
+        "prefill_ragged_batches": prefill_ragged_bench(dev),
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(w)

@@ -346,3 +346,33 @@ def test_check_plan_flag_defaults_to_the_environment(monkeypatch):
     monkeypatch.setenv("AICOMP_CHECK_PLANS", "1")
     assert StepPlanner(num_blocks=8, device="cpu").check_plans is True
     assert StepPlanner(num_blocks=8, device="cpu", check_plans=False).check_plans is False
+
+
+def test_prefill_item_list_names_every_tile_once_most_expensive_first():
+    """ops.prefill_items: the order a planner hands to the prefill kernel.  Every query tile that has
+    rows appears exactly once (also for a chunk longer than its context, whose rows the kernel zeroes),
+    costs (keys of the tile's last row) never rise along the list, and a launch that is resident all
+    at once gets its second round from the cheap end."""
+    from aicomp_amd import ops
+    rng = np.random.default_rng(3)
+    for trial in range(50):
+        S = int(rng.integers(1, 40))
+        new = rng.choice([0, 1, 7, 31, 32, 33, 64, 100, 512], size=S)
+        prior = rng.integers(0, 3000, size=S)
+        ctx = prior + new
+        if trial % 7 == 0 and S > 1:
+            ctx[1] = max(0, new[1] - 5)                                   # an inconsistent row
+        tile = int(rng.choice([8, 16, 32, 64, 128]))
+        items = ops.prefill_items(ctx, new, tile)
+        want = {(s, q) for s in range(S) for q in range(-(-int(new[s]) // tile))}
+        got = [tuple(x) for x in items.tolist()]
+        assert len(got) == len(set(got)) and set(got) == want, trial
+        keys = [min(ctx[s], ctx[s] - new[s] + (q + 1) * tile) for s, q in got]
+        assert all(a >= b for a, b in zip(keys, keys[1:])), trial
+        assert items.dtype == np.int32 and items.shape == (len(want), 2)
+    # 512 workgroups on 256 CUs, 8 per item: 32 items per round; the second round runs cheap to expensive
+    items = ops.prefill_items([2048], [2048], 32, num_head_groups=8, num_cus=256)
+    assert items[:32, 1].tolist() == list(range(63, 31, -1)) and items[32:, 1].tolist() == list(range(0, 32))
+    # a larger launch is dispatched as places free up: expensive first throughout
+    items = ops.prefill_items([4096], [4096], 32, num_head_groups=8, num_cus=256)
+    assert items[:, 1].tolist() == list(range(127, -1, -1))

@@ -308,3 +308,39 @@ def test_long_prompt_all_rows_and_scaling_in_v(device):
     want = orc.paged_prefill_attn(raw(c["q"]), raw(kp), raw(vp), c["table"].cpu().numpy(), [n], [0, n], c["scale"],
                                   "bf16", "bf16", gather=orc.gather_context_fast)
     assert_close_attn(to_f64(got), want, BF16_ATOL, BF16_RTOL, "4096-token prompt, all rows")
+
+
+# ------------------------------------------------------------------ caller-ranked item lists
+@pytest.mark.parametrize("dtype,kv,d,hq,hkv", [(torch.bfloat16, None, 128, 32, 8), (torch.bfloat16, None, 64, 8, 2),
+                                               (torch.bfloat16, torch.float8_e4m3fn, 128, 16, 2),
+                                               (torch.float16, None, 128, 6, 2), (torch.float32, None, 128, 8, 2),
+                                               (torch.float32, None, 64, 4, 4), (torch.bfloat16, None, 256, 4, 1)])
+def test_prefill_with_a_caller_ranked_item_list_equals_grid_order(device, dtype, kv, d, hq, hkv):
+    """aicomp_paged_prefill_attn_items: the same launch with its (sequence, query tile) pairs in the
+    order a planner ranks them.  Bit for bit the result of the plain call, on ragged chunk batches
+    (lengths 1 to 300, priors 0 to 700, an empty chunk), for every kernel that takes a list, with
+    chunk bounds that select one and two column groups per wave; pairs that name no sequence or no
+    tile are skipped; a kernel that takes no list (head_dim 256) ignores it."""
+    priors = [0, 700, 33, 5, 0, 310, 64, 1, 200, 17]
+    for news in ([300, 1, 40, 130, 0, 64, 17, 2, 96, 33], [20, 1, 16, 7, 0, 3, 17, 2, 9, 12]):
+        c = build_case(device, priors, news, hq, hkv, d, dtype=dtype, kv_dtype=kv, seed=len(news) + d)
+        plain = run(c, max_q_len=max(news))
+        tile = ops.prefill_tile_positions(hq, hkv, d, 16, dtype, c["k_pool"].dtype, max(news))
+        assert (tile == 0) == (d == 256)
+        items = ops.prefill_items(c["ctx_list"], news, tile or 32, num_head_groups=hq // (hq // hkv), num_cus=256)
+        junk = np.array([[-1, 0], [len(news), 0], [0, 1000], [3, -2]], dtype=np.int32)
+        items = np.concatenate([junk[:2], items, junk[2:]])
+        out = torch.full_like(c["q"], float("nan"))
+        ops.paged_prefill_attn(out, c["q"], c["k_pool"], c["v_pool"], c["table"], c["ctx"], c["cu"], c["scale"],
+                               max_q_len=max(news), k_scale=c["ks"], v_scale=c["vs"],
+                               items=torch.from_numpy(items).to(device))
+        torch.cuda.synchronize()
+        bits = lambda t: t.view(torch.int16) if t.element_size() == 2 else t
+        assert torch.equal(bits(out), bits(plain)), (dtype, kv, d, news[0])
+    # the registered operator takes the same list
+    t = __import__("aicomp_amd")._lib.torch_ops()
+    out2 = torch.full_like(c["q"], float("nan"))
+    t.paged_prefill_attn(out2, c["q"], c["k_pool"], c["v_pool"], c["table"], c["ctx"], c["cu"], c["scale"], max(news),
+                         c["ks"], c["vs"], torch.from_numpy(items).to(device))
+    torch.cuda.synchronize()
+    assert torch.equal(bits(out2), bits(plain))
