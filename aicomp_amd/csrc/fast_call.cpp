@@ -2,7 +2,7 @@
 // from CachedScaledDotProductAttention.forward (opt_prime/opt_prime/kv_cache.py:340-403) into
 // aicomp_paged_decode_attn_append.  The reference's own engine decodes at batch 1
 // (inference.py:1036-1044), where the GPU needs 5 to 8 us per call and every microsecond of host
-// time is step time.  torch.ops.mi355_kv.decode_step (torch_ops.cpp) spends about two of its six
+// time is step time.  torch.ops.mi355_kv.decode_step (torch_ops.cpp) spends about three of its eight
 // microseconds in the dispatcher and in re-checking tensors that never change between steps; here
 // a layer's pools, table and context-length rows are checked once and kept in a capsule, and a
 // step is one METH_FASTCALL function: three tensors unpacked, the output allocated, one C call.
@@ -14,6 +14,7 @@
 #include <Python.h>
 
 #include <ATen/ATen.h>
+#include <ATen/hip/EmptyTensor.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/csrc/autograd/python_variable.h>
 
@@ -142,7 +143,8 @@ PyObject* decode_step(PyObject*, PyObject* const* args, Py_ssize_t nargs) {
             ws = t.data_ptr();
             ws_bytes = (size_t)t.numel();
         }
-        at::Tensor out = at::empty(query.sizes(), query.options());
+        // (the allocator's own entry: at::empty goes through the dispatcher for the same result)
+        at::Tensor out(at::detail::empty_cuda(query.sizes(), L->st, L->dev, c10::MemoryFormat::Contiguous));
         const int rc = aicomp_paged_decode_attn_append(
             out.data_ptr(), query.data_ptr(), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1) * hstep, L->kp, L->vp,
             L->table, L->table_stride, L->ctx + (position + 1) * L->ctx_stride, L->B, hq, L->hkv, L->d, L->bs, width,

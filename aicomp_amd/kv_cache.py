@@ -527,6 +527,18 @@ class CachedScaledDotProductAttention(nn.Module):
                 or _nn_module._global_forward_hooks or _nn_module._global_forward_pre_hooks
                 or _nn_module._global_backward_hooks or _nn_module._global_backward_pre_hooks):
             return super().__call__(*args, **kwargs)
+        if len(args) == 3 and not kwargs:
+            # the generation loop's own call, attn(query, key, value) on a decode step: same route
+            # as in forward() below, one Python frame less
+            store = self._store
+            if (store is not None and store._fast is not None and _route == "fast" and self._enabled
+                    and self.kv_manager is None and not self._device_positions):
+                query, key, value = args
+                pos = self.cache_pos
+                if query.dim() == 4 and query.shape[2] == 1 and key.dtype == store.dtype and pos < self.max_seq_len:
+                    out = _FAST.decode_step(store._fast, query, key, value, pos, self._group, store.default_scale)
+                    self.__dict__["cache_pos"] = pos + 1      # (nn.Module.__setattr__ costs 0.5 us; a plain int needs none of it)
+                    return out
         return self.forward(*args, **kwargs)
 
     def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
@@ -543,7 +555,7 @@ class CachedScaledDotProductAttention(nn.Module):
                 out = _FAST.decode_step(store._fast, query, key, value, pos, self._group,
                                         store.default_scale if not kwargs or kwargs.get("scale") is None
                                         else float(kwargs["scale"]))
-                self.cache_pos = pos + 1
+                self.__dict__["cache_pos"] = pos + 1
                 return out
         if not self._enabled:
             return F.scaled_dot_product_attention(query, key, value, attn_mask=attn_mask,
@@ -561,7 +573,7 @@ class CachedScaledDotProductAttention(nn.Module):
             if n == 1:                            # decode step: one fused call, as in internal mode
                 out = self.kv_manager.decode_step(self.layer_idx, query, key, value, pos, scale)
                 if out is not None:
-                    self.cache_pos = pos + 1
+                    self.__dict__["cache_pos"] = pos + 1
                     return out
             store, _, _ = self.kv_manager.append(self.layer_idx, key, value, position=pos)
         else:
@@ -590,7 +602,7 @@ class CachedScaledDotProductAttention(nn.Module):
                 # recorded into a graph executes nothing: the host position stays (see advance()).
                 out = store.decode_step(query, key, value, pos, self._group, scale, live=self._device_positions)
                 if not (self._device_positions and torch.cuda.is_current_stream_capturing()):
-                    self.cache_pos = pos + 1      # only after the call was accepted
+                    self.__dict__["cache_pos"] = pos + 1      # only after the call was accepted
                 return out
             store.append(key, value, pos, self._group)
         self.cache_pos = pos + n

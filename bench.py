@@ -456,8 +456,8 @@ def mixed_step_bench(dev, reps=40):
 def host_cost_bench(dev):
     """Host time of ONE decode call of the drop-in operator at the size the reference's own engine
     runs (batch 1, Llama-3.2-1B heads: 32 / 8, head_dim 64, bf16, K/V arriving expanded by
-    repeat_kv): the Python thread's time per call, timed over 1000 calls without a synchronisation
-    inside (the position is set back before every call, so each call sees the stated context).
+    repeat_kv): the Python thread's time per call, timed over 1024 calls without a synchronisation
+    inside (32 consecutive steps from the stated context, then the position is set back).
     At 600 cached tokens the call is one launch (whole rows), at 1500 two (256-token partitions and
     their merge).  Through each host route to the same C entry point: the CPython function over a
     per-layer handle (the one the operator takes), the registered operator
@@ -485,11 +485,12 @@ def host_cost_bench(dev):
                 torch.cuda.synchronize()
                 best = None
                 for _ in range(5):
-                    n = 1000
+                    n = 1024
                     t0 = time.perf_counter()
-                    for _ in range(n):
-                        op.cache_pos = ctx
-                        op(q, k, v)
+                    for _ in range(n // 32):
+                        op.cache_pos = ctx                    # 32 steps from the stated context, then back
+                        for _ in range(32):
+                            op(q, k, v)
                     host = (time.perf_counter() - t0) / n
                     torch.cuda.synchronize()
                     best = host if best is None else min(best, host)
