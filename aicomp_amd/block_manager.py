@@ -22,7 +22,8 @@ kernels read (``block_table``, ``context_lens``, ``slot_mapping``,
 Row order inside a plan: sequences that ingest more than one token (prompt
 chunks) first, then the one-token sequences; ``paged_attention_step`` below
 runs the append, the chunked-prefill kernel on the first group and the decode
-kernel on the second.
+kernel on the second, or, for a mixed step with a moderate decode part, one
+launch of the chunked-prefill kernel over both (``StepPlan.step_items``).
 
 Token t of a sequence lives in slot ``block_table[t // BS] * BS + t % BS``.
 """
@@ -208,6 +209,45 @@ class StepPlan:
         if key not in self._prefill_items:
             cus = torch.cuda.get_device_properties(query.device).multi_processor_count if query.is_cuda else 0
             items = ops.prefill_items(self.host_context_lens[:npre], self.new_lens[:npre], tile, hgroups, cus)
+            self._prefill_items[key] = torch.from_numpy(items).to(query.device, non_blocking=True)
+        return self._prefill_items[key]
+
+    # Longest decode row and largest decode batch for which a mixed step goes through one launch
+    # (measured on MI355X, 32 / 8 and 64 / 8 heads, head_dim 64 and 128, 1 to 16 chunks of 128 to
+    # 2048 tokens with 16 to 250 rows: within these bounds the one launch takes 0.95 to 1.65 times
+    # less than chunks and rows through their own kernels, 1.06 on 4 x 512 + 60 rows of up to 4096
+    # tokens; a row of 8192 and more tokens, walked by a single workgroup row, makes it up to
+    # twice as slow, and beyond ~128 rows the decode kernel's faster streaming wins)
+    ONE_LAUNCH_MAX_CONTEXT = 4608
+    ONE_LAUNCH_MAX_ROWS = 128
+
+    def step_items(self, query: torch.Tensor, k_pool: torch.Tensor) -> Optional[torch.Tensor]:
+        """Item list over ALL sequences of a mixed step (chunks and one-token rows) for one launch
+        of the chunked-prefill kernel, or ``None`` when the step should go through the prefill
+        and decode kernels separately: no chunk or no decode row in it, pools of another type
+        than the 16-bit queries, a kernel that takes no list, a chunk bound too short for the
+        two-column-group kernel, or a decode part outside the bounds above.  Cached per step."""
+        from . import ops
+        npre, ndec = self.num_prefill_seqs, self.num_decode_seqs
+        if not npre or not ndec or ndec > self.ONE_LAUNCH_MAX_ROWS:
+            return None
+        if query.dtype not in (torch.bfloat16, torch.float16) or k_pool.dtype != query.dtype:
+            return None
+        if int(self.host_context_lens[npre:].max()) > self.ONE_LAUNCH_MAX_CONTEXT:
+            return None
+        hq, hkv, d, bs = query.shape[1], k_pool.shape[1], k_pool.shape[3], k_pool.shape[2]
+        tile = ops.prefill_tile_positions(hq, hkv, d, bs, query.dtype, k_pool.dtype, self.max_q_len)
+        group = hq // hkv
+        gpack = group if 16 % group == 0 else 1
+        if tile * gpack != 128:                   # (0: no list; 64: the one-column-group kernel)
+            return None
+        hgroups = hq // gpack
+        key = ("step", tile, hgroups, query.device)
+        if self._prefill_items is None:
+            self._prefill_items = {}
+        if key not in self._prefill_items:
+            cus = torch.cuda.get_device_properties(query.device).multi_processor_count if query.is_cuda else 0
+            items = ops.step_items(self.host_context_lens, self.new_lens, npre, tile, hgroups, cus)
             self._prefill_items[key] = torch.from_numpy(items).to(query.device, non_blocking=True)
         return self._prefill_items[key]
 
@@ -563,13 +603,23 @@ def paged_attention_step(plan: StepPlan, out: torch.Tensor, query: torch.Tensor,
 
     ``query`` / ``out`` are ``[T, Hq, D]``, ``key`` / ``value`` ``[T, Hkv, D]`` in the plan's
     row order (``cu_q_lens``).  The prompt chunks go through the chunked-prefill kernel;
-    the one-token rows go through the decode kernel with their append fused into it.
+    the one-token rows go through the decode kernel with their append fused into it, or, in a
+    mixed step whose decode part is small enough (``StepPlan.step_items``), through the same
+    launch as the chunks.
     Replaces, per sequence, the append + ``.contiguous()`` + SDPA of
     opt_prime/opt_prime/kv_cache.py:385-415.
     """
     from . import ops
     npre, S = plan.num_prefill_seqs, plan.num_seqs
     t_pre = plan.num_prefill_tokens
+    items = plan.step_items(query, k_pool)
+    if items is not None:
+        # mixed step, decode part within the measured bounds: every new row appended, then one
+        # launch over all sequences (a decode row is a chunk of one token)
+        ops.kv_append(key, value, k_pool, v_pool, plan.slot_mapping, k_scale, v_scale)
+        return ops.paged_prefill_attn(out, query, k_pool, v_pool, plan.block_table, plan.context_lens,
+                                      plan.cu_q_lens, scale, max_q_len=plan.max_q_len, k_scale=k_scale,
+                                      v_scale=v_scale, items=items)
     if npre:
         ops.kv_append(key[:t_pre], value[:t_pre], k_pool, v_pool, plan.slot_mapping[:t_pre], k_scale, v_scale)
         ops.paged_prefill_attn(out[:t_pre], query[:t_pre], k_pool, v_pool, plan.block_table[:npre],

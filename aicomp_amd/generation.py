@@ -79,6 +79,10 @@ class PagedAttentionBackend:
         ops.rope_kv_append(query, key, value, self.cos, self.sin, plan.positions, kp, vp, plan.slot_mapping,
                            ks, vs, query_out=q)
         npre, S, t_pre = plan.num_prefill_seqs, plan.num_seqs, plan.num_prefill_tokens
+        items = plan.step_items(q, kp)
+        if items is not None:                      # mixed step: chunks and decode rows in one launch
+            return ops.paged_prefill_attn(out, q, kp, vp, plan.block_table, plan.context_lens, plan.cu_q_lens,
+                                          self.scale, max_q_len=plan.max_q_len, k_scale=ks, v_scale=vs, items=items)
         if npre:
             ops.paged_prefill_attn(out[:t_pre], q[:t_pre], kp, vp, plan.block_table[:npre], plan.context_lens[:npre],
                                    plan.cu_q_lens[:npre + 1], self.scale, max_q_len=plan.max_q_len,

@@ -376,3 +376,64 @@ def test_prefill_item_list_names_every_tile_once_most_expensive_first():
     # a larger launch is dispatched as places free up: expensive first throughout
     items = ops.prefill_items([4096], [4096], 32, num_head_groups=8, num_cus=256)
     assert items[:, 1].tolist() == list(range(127, -1, -1))
+
+
+def _mixed_plan(ctx, new, npre, max_q):
+    import torch
+    from aicomp_amd.block_manager import StepPlan
+    S = len(ctx)
+    cu = np.concatenate([[0], np.cumsum(new)]).astype(np.int32)
+    return StepPlan(seq_ids=list(range(S)), num_prefill_seqs=npre, new_lens=np.asarray(new, dtype=np.int32), max_q_len=max_q,
+                    total_new_tokens=int(cu[-1]), block_table=torch.zeros(S, 1, dtype=torch.int32),
+                    context_lens=torch.tensor(ctx, dtype=torch.int32), cu_q_lens=torch.from_numpy(cu),
+                    slot_mapping=None, positions=None, preempted=[], host_context_lens=np.asarray(ctx), host_cu_q_lens=cu)
+
+
+def test_step_item_list_orders_a_mixed_step_for_one_launch():
+    """ops.step_items: every chunk tile and every decode row exactly once; decode rows that are the
+    longer items open the list (one CU-round of them, then one of chunk tiles, then alternating,
+    each kind longest first); shorter decode rows leave the list in falling cost."""
+    from aicomp_amd import ops
+    rng = np.random.default_rng(5)
+    npre, ndec, tile = 4, 60, 32
+    new = [512] * npre + [1] * ndec
+    ctx = [int(p) + 512 for p in rng.integers(0, 2049, npre)] + [int(c) for c in rng.integers(513, 4098, ndec)]
+    items = ops.step_items(ctx, new, npre, tile, num_head_groups=8, num_cus=256)
+    want = {(s, q) for s in range(npre) for q in range(16)} | {(s, 0) for s in range(npre, npre + ndec)}
+    got = [tuple(x) for x in items.tolist()]
+    assert len(got) == len(set(got)) and set(got) == want and items.dtype == np.int32
+    assert all(s >= npre for s, _ in got[:32]) and all(s < npre for s, _ in got[32:64])
+    dec_keys = [ctx[s] for s, _ in got if s >= npre]
+    assert dec_keys == sorted(dec_keys, reverse=True)                       # each kind longest first
+    pre_keys = [min(ctx[s], ctx[s] - 512 + (q + 1) * tile) for s, q in got if s < npre]
+    assert pre_keys == sorted(pre_keys, reverse=True)
+    kinds = [s >= npre for s, _ in got[64:64 + 2 * min(ndec - 32, 64 - 32)]]
+    assert kinds == [True, False] * (len(kinds) // 2)                       # then alternating
+    # short decode rows: falling cost over both kinds
+    ctx2 = ctx[:npre] + [int(c) for c in rng.integers(2, 300, ndec)]
+    items2 = ops.step_items(ctx2, new, npre, tile, num_head_groups=8, num_cus=256)
+    keys2 = [min(ctx2[s], ctx2[s] - new[s] + (q + 1) * tile) for s, q in items2.tolist()]
+    assert keys2 == sorted(keys2, reverse=True) and {tuple(x) for x in items2.tolist()} == want
+    # no decode rows, or no chunks: the chunk order
+    assert (ops.step_items(ctx[:npre], new[:npre], npre, tile, 8, 256) == ops.prefill_items(ctx[:npre], new[:npre], tile, 8, 0)).all()
+
+
+def test_step_plan_sends_only_moderate_decode_parts_through_one_launch():
+    """StepPlan.step_items: a list for a mixed step of 16-bit pools whose decode part is within
+    the measured bounds, None otherwise (the step then goes through the prefill and decode kernels)."""
+    import torch
+    q = torch.zeros(1, 32, 128, dtype=torch.bfloat16)
+    pool = torch.zeros(1, 8, 16, 128, dtype=torch.bfloat16)
+    mixed = lambda ctx_dec, n_dec=8, chunk=512, npre=2: _mixed_plan([chunk + 100] * npre + [ctx_dec] * n_dec,
+                                                                   [chunk] * npre + [1] * n_dec, npre, chunk)
+    it = mixed(2000).step_items(q, pool)
+    assert it is not None and it.shape == (2 * 16 + 8, 2)
+    plan = mixed(2000)
+    assert plan.step_items(q, pool) is plan.step_items(q, pool)                           # built once per step
+    assert mixed(4608).step_items(q, pool) is not None and mixed(4609).step_items(q, pool) is None   # a long decode row
+    assert mixed(2000, n_dec=128).step_items(q, pool) is not None and mixed(2000, n_dec=129).step_items(q, pool) is None
+    assert mixed(2000, npre=0).step_items(q, pool) is None and mixed(2000, n_dec=0).step_items(q, pool) is None
+    assert mixed(2000).step_items(q, pool.to(torch.float8_e4m3fn)) is None                # fp8 pools: own kernels
+    assert mixed(2000).step_items(q.float(), pool.float()) is None
+    assert mixed(2000, chunk=16).step_items(q, pool) is None                              # one-column-group kernel
+    assert mixed(2000).step_items(torch.zeros(1, 32, 256, dtype=torch.bfloat16), torch.zeros(1, 8, 16, 256, dtype=torch.bfloat16)) is None

@@ -95,8 +95,27 @@ def test_full_chunked_prefill_mixed(device):
                                   w.ctx_list[:npre], w.cu_q_lens.cpu().numpy()[:npre + 1], w.scale, "bf16", "bf16",
                                   gather=orc.gather_context_fast)
     assert_close_attn(to_f64(out), want, BF16_ATOL, BF16_RTOL, "all prefill rows of the mixed step")
-    want = oracle_decode_all(w, w.query[T:], w.block_table[npre:], w.ctx_list[npre:])
-    assert_close_attn(to_f64(dec), want, BF16_ATOL, BF16_RTOL, "all decode rows of the mixed step")
+    want_dec = oracle_decode_all(w, w.query[T:], w.block_table[npre:], w.ctx_list[npre:])
+    assert_close_attn(to_f64(dec), want_dec, BF16_ATOL, BF16_RTOL, "all decode rows of the mixed step")
+    # the same step the way a planner's attention call runs it: this decode part is within the
+    # bounds for ONE launch of the chunked-prefill kernel over chunks and decode rows alike.
+    # Chunk rows bit for bit those of the chunks-only call (an item runs the same code wherever
+    # it stands in the list), decode rows against the oracle.
+    from aicomp_amd.block_manager import StepPlan, paged_attention_step
+    plan = StepPlan(seq_ids=list(range(w.num_seqs)), num_prefill_seqs=npre, new_lens=np.asarray(w.new_list, dtype=np.int32),
+                    max_q_len=512, total_new_tokens=int(w.query.shape[0]), block_table=w.block_table,
+                    context_lens=w.context_lens, cu_q_lens=w.cu_q_lens, slot_mapping=w.slot_mapping, positions=None,
+                    preempted=[], host_context_lens=np.asarray(w.ctx_list), host_cu_q_lens=w.cu_q_lens.cpu().numpy())
+    items = plan.step_items(w.query, w.k_pool)
+    assert items is not None and items.shape == (4 * 16 + 60, 2)
+    assert sorted(map(tuple, items.cpu().tolist())) == sorted([(s, q) for s in range(4) for q in range(16)] +
+                                                              [(s, 0) for s in range(4, 64)])
+    out_all = torch.full_like(w.query, float("nan"))
+    paged_attention_step(plan, out_all, w.query, w.new_key, w.new_value, w.k_pool, w.v_pool, w.scale)
+    torch.cuda.synchronize()
+    assert torch.equal(out_all[:T].view(torch.int16), out.view(torch.int16))
+    assert_close_attn(to_f64(out_all[T:]), want_dec, BF16_ATOL, BF16_RTOL, "decode rows of the mixed step, one launch")
+    assert torch.equal(before_k.view(torch.int16), w.k_pool.view(torch.int16))       # the append wrote the same rows again
 
 
 def test_full_fp32_anchor_vs_cpu_reference_path(device):
