@@ -78,6 +78,20 @@ def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
+def plan_of_workload(w):
+    """The workload's step as the plan a StepPlanner would hand to paged_attention_step (chunks
+    first, one-token rows after; the workload's own tables and lengths)."""
+    import numpy as np
+    from aicomp_amd.block_manager import StepPlan
+    npre = w.num_prefill_seqs
+    return StepPlan(seq_ids=list(range(w.num_seqs)), num_prefill_seqs=npre,
+                    new_lens=np.asarray(w.new_list, dtype=np.int32),
+                    max_q_len=max(w.new_list[:npre]) if npre else 0, total_new_tokens=int(w.query.shape[0]),
+                    block_table=w.block_table, context_lens=w.context_lens, cu_q_lens=w.cu_q_lens,
+                    slot_mapping=w.slot_mapping, positions=None, preempted=[],
+                    host_context_lens=np.asarray(w.ctx_list), host_cu_q_lens=w.cu_q_lens.cpu().numpy())
+
+
 def run_decode_config(name, steps, warmup, dev):
     """Append + decode for one workload; returns timing and algorithmic figures."""
     import torch
@@ -164,14 +178,8 @@ def run_decode_config(name, steps, warmup, dev):
         # decides between one launch over all sequences and chunks / decode rows through their own
         # kernels), over the same rotating pools; the three-launch loop above stays for the
         # per-kernel figures.
-        import numpy as np
-        from aicomp_amd.block_manager import StepPlan, paged_attention_step
-        host_ctx = w.context_lens.cpu().numpy()
-        plan = StepPlan(seq_ids=list(range(S)), num_prefill_seqs=npre, new_lens=np.asarray(w.new_list, dtype=np.int32),
-                        max_q_len=max_q, total_new_tokens=int(w.query.shape[0]), block_table=w.block_table,
-                        context_lens=w.context_lens, cu_q_lens=w.cu_q_lens, slot_mapping=w.slot_mapping,
-                        positions=None, preempted=[], host_context_lens=host_ctx,
-                        host_cu_q_lens=w.cu_q_lens.cpu().numpy())
+        from aicomp_amd.block_manager import paged_attention_step
+        plan = plan_of_workload(w)
         out_all = torch.empty_like(w.query)
         one_launch = plan.step_items(w.query, w.k_pool) is not None
 
@@ -807,6 +815,17 @@ def profile_target(which, steps, warmup, dev, settle_ms=30.0):
         torch.cuda.synchronize()
         print(f"{which}: {warmup + steps} replays of a graph of 3 mixed steps ({how})")
         return
+    if which == "mixed_planned":
+        # the named mixed step the way paged_attention_step runs it (one pool)
+        from aicomp_amd.block_manager import paged_attention_step
+        w = workloads.make_workload("chunked_prefill_mixed", device=dev)
+        plan = plan_of_workload(w)
+        out = torch.empty_like(w.query)
+        one = plan.step_items(w.query, w.k_pool) is not None
+        how = drive(lambda: paged_attention_step(plan, out, w.query, w.new_key, w.new_value, w.k_pool, w.v_pool, w.scale))
+        print(f"mixed_planned (chunked_prefill_mixed): {how}; "
+              f"{'append + one launch over chunks and decode rows' if one else 'append + prefill + decode kernels'}")
+        return
     if which == "prefill_long":
         # one fresh prompt of 8192 tokens at the Llama-3-8B head shape (a row of prefill_other_shapes)
         import math
@@ -953,7 +972,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     ap.add_argument("--only", choices=["decode", "append", "copy", "prefill", "prefill_long", "decode_fp8", "decode_long", "decode_d64", "rope", "sample",
-                             "mixed_serial", "mixed_streams"],
+                             "mixed_serial", "mixed_streams", "mixed_planned"],
                     help="profiling target: launch just this kernel --steps times (no JSON line)")
     ap.add_argument("--settle-ms", type=float, default=30.0,
                     help="with --only: untimed launches for this long before the timed ones")
