@@ -60,6 +60,7 @@ try:
     _TORCH_DECODE = _lib.torch_ops().decode_step.default
 except _lib.LibraryMissing:
     _TORCH_DECODE = None
+_PLAIN_KWARGS = frozenset(("attn_mask", "dropout_p", "is_causal"))      # keywords that leave a decode call as it is
 _route = "fast" if _FAST is not None else ("torch_op" if _TORCH_DECODE is not None else "ctypes")
 
 
@@ -527,9 +528,11 @@ class CachedScaledDotProductAttention(nn.Module):
                 or _nn_module._global_forward_hooks or _nn_module._global_forward_pre_hooks
                 or _nn_module._global_backward_hooks or _nn_module._global_backward_pre_hooks):
             return super().__call__(*args, **kwargs)
-        if len(args) == 3 and not kwargs:
-            # the generation loop's own call, attn(query, key, value) on a decode step: same route
-            # as in forward() below, one Python frame less
+        if len(args) == 3 and (not kwargs or (kwargs.keys() <= _PLAIN_KWARGS and not kwargs.get("dropout_p"))):
+            # the model's own call on a decode step, attn(query, key, value, attn_mask=..., dropout_p=0.0,
+            # is_causal=...) as compiler_fx/modeling_llama.py:607-614 issues it (the mask and the causal
+            # flag of a one-token call change nothing, kv_cache.py:397-403): same route as in forward()
+            # below, one Python frame less
             store = self._store
             if (store is not None and store._fast is not None and _route == "fast" and self._enabled
                     and self.kv_manager is None and not self._device_positions):

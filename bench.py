@@ -515,7 +515,8 @@ def host_cost_bench(dev):
     B, hq, g, d = 1, 32, 4, 64
     hkv = hq // g
     mk = lambda n, h: torch.randn(B, h, n, d, device=dev).to(torch.bfloat16)
-    res = {"shape": "batch 1, 32 query / 8 KV heads (K/V expanded to 32), head_dim 64, bf16"}
+    res = {"shape": "batch 1, 32 query / 8 KV heads (K/V expanded to 32), head_dim 64, bf16",
+           "call": "op(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False)"}
     available = {"fast": akv._FAST is not None, "torch_op": akv._TORCH_DECODE is not None, "ctypes": True}
     for name in ("fast", "torch_op", "ctypes"):
         if not available[name]:
@@ -529,7 +530,7 @@ def host_cost_bench(dev):
             for ctx in (600, 1500):
                 for _ in range(200):
                     op.cache_pos = ctx
-                    op(q, k, v)
+                    op(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False)
                 torch.cuda.synchronize()
                 best = None
                 for _ in range(5):
@@ -537,8 +538,8 @@ def host_cost_bench(dev):
                     t0 = time.perf_counter()
                     for _ in range(n // 32):
                         op.cache_pos = ctx                    # 32 steps from the stated context, then back
-                        for _ in range(32):
-                            op(q, k, v)
+                        for _ in range(32):                   # the call as compiler_fx/modeling_llama.py:607-614 issues it
+                            op(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False)
                     host = (time.perf_counter() - t0) / n
                     torch.cuda.synchronize()
                     best = host if best is None else min(best, host)

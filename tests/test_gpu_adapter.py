@@ -283,3 +283,36 @@ def test_device_positions_survive_a_rejected_call_and_a_forgotten_advance(device
     used = op._store.slot_table[:, :24].reshape(-1)
     flat = lambda p: p.permute(0, 2, 1, 3).reshape(-1, p.shape[1], p.shape[3])
     assert torch.equal(flat(op._store.k_pool)[used].view(torch.int16), flat(before)[used].view(torch.int16))
+
+
+def test_decode_call_styles_agree(device, host_route):
+    """The operator's decode call as a model issues it (three positionals and attn_mask / dropout_p /
+    is_causal keywords, compiler_fx/modeling_llama.py:607-614), with positionals only, and with a
+    keyword the short route does not take (scale): same cache, same positions, bit-identical output
+    where the arguments mean the same, and the scale honoured where it is given."""
+    B, hq, g, d = 2, 8, 4, 64
+    hkv = hq // g
+    torch.manual_seed(11)
+    mk = lambda n, h: (torch.randn(B, h, n, d, device=device) * 0.7).to(torch.bfloat16)
+    ex = lambda x: x.repeat_interleave(g, 1)
+    ops_ = [akv.CachedScaledDotProductAttention(0, 64, num_kv_groups=g) for _ in range(4)]
+    for o in ops_:
+        o.enable()
+    q, k, v = mk(9, hq), mk(9, hkv), mk(9, hkv)
+    for o in ops_:
+        o(q, ex(k), ex(v), is_causal=True)
+    for step in range(3):
+        q, k, v = mk(1, hq), mk(1, hkv), mk(1, hkv)
+        a = ops_[0](q, ex(k), ex(v))
+        b = ops_[1](q, ex(k), ex(v), attn_mask=None, dropout_p=0.0, is_causal=False)
+        c = ops_[2](q, ex(k), ex(v), attn_mask=torch.ones(1, 1, 1, 10 + step, dtype=torch.bool, device=device), is_causal=True)
+        e = ops_[3](q, ex(k), ex(v), scale=1 / math.sqrt(d))
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16)) and torch.equal(a.view(torch.int16), c.view(torch.int16))
+        assert torch.equal(a.view(torch.int16), e.view(torch.int16))
+        assert [o.cache_pos for o in ops_] == [10 + step] * 4
+    with pytest.raises(ValueError):
+        ops_[0](q, ex(k), ex(v), dropout_p=0.1)
+    assert ops_[0].cache_pos == 12                                   # a refused call stores nothing
+    half = ops_[3](q, ex(k), ex(v), scale=0.5 / math.sqrt(d))
+    full = ops_[2](q, ex(k), ex(v))
+    assert not torch.equal(half.view(torch.int16), full.view(torch.int16))
