@@ -7,4 +7,4 @@
 from . import _lib  # noqa: F401
 
 __all__ = ["ops", "kv_cache", "workloads"]
-__version__ = "0.1.0"
+__version__ = "0.2.0"

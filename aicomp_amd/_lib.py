@@ -30,6 +30,7 @@ SYMBOLS = (
 )
 
 F32, BF16, FP8_E4M3, F16 = 0, 1, 2, 3
+MIN_VERSION = 200            # 0.2.0: the entry points of SYMBOLS above
 
 _lock = threading.RLock()       # torch_ops() loads the HIP library while holding it
 _lib = None
@@ -96,6 +97,9 @@ def load() -> C.CDLL:
                 if not hasattr(lib, s):
                     raise LibraryMissing(f"{LIB_PATH} does not export {s}")
             _declare(lib)
+            if lib.aicomp_kv_version() < MIN_VERSION:
+                raise LibraryMissing(f"{LIB_PATH} is version {lib.aicomp_kv_version()}, this package needs "
+                                     f">= {MIN_VERSION}: rebuild it with `python -m aicomp_amd.build`")
             _lib = lib
         return _lib
 

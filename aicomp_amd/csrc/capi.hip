@@ -105,7 +105,7 @@ using namespace aicomp;
 
 extern "C" {
 
-int aicomp_kv_version(void) { return 100; }
+int aicomp_kv_version(void) { return 200; }
 
 const char* aicomp_kv_last_error(void) { return g_err; }
 

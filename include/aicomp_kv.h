@@ -46,7 +46,9 @@ extern "C" {
 #define AICOMP_KV_FP8_E4M3  2       /* OCP e4m3 ("e4m3fn"), max finite 448       */
 #define AICOMP_KV_F16       3       /* IEEE binary16                             */
 
-/* Library version (major*10000 + minor*100 + patch). */
+/* Library version (major*10000 + minor*100 + patch).  200 = 0.2.0: added
+ * aicomp_kv_set_small_decode_tokens, aicomp_paged_prefill_attn_items and
+ * aicomp_paged_prefill_tile_positions; every 0.1 entry point is unchanged. */
 int aicomp_kv_version(void);
 
 /* Message of the last failing call on this thread ("" if none). */
