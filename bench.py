@@ -92,8 +92,15 @@ def plan_of_workload(w):
                     host_context_lens=np.asarray(w.ctx_list), host_cu_q_lens=w.cu_q_lens.cpu().numpy())
 
 
-def run_decode_config(name, steps, warmup, dev):
-    """Append + decode for one workload; returns timing and algorithmic figures."""
+def run_decode_config(name, steps, warmup, dev, settle_ms=30.0):
+    """Append + decode for one workload; returns timing and algorithmic figures.
+
+    Clock protocol: an idle MI355X takes about 30 ms of continuous work to bring its shader clock
+    up, and the launches in between run up to 10-15 % slower (6 % on the Llama-3.2-1B shape, 3 % on
+    the headline shape, whose kernel waits for HBM most of the time).  A serving process never sees
+    that ramp after its first step, so every timed loop here is preceded by `settle_ms` of the same
+    steps, untimed, before the `warmup` steps; the same K steps timed from an idle part (only the
+    `warmup` steps before them) are kept beside the figure as `from_idle`."""
     import torch
     from aicomp_amd import ops, workloads
     w = workloads.make_workload(name, device=dev)
@@ -146,11 +153,22 @@ def run_decode_config(name, steps, warmup, dev):
     def append_only():
         ops.kv_append(w.new_key, w.new_value, w.k_pool, w.v_pool, w.slot_mapping, w.k_scale, w.v_scale)
 
-    def timed_loop(rotate):
+    def settle(fn):
+        """Untimed steps for settle_ms (a synchronisation every 8 steps keeps the queue short)."""
+        t0, i = time.perf_counter(), 0
+        while (time.perf_counter() - t0) * 1e3 < settle_ms:
+            for _ in range(8):
+                fn(i)
+                i += 1
+            torch.cuda.synchronize()
+
+    def timed_loop(rotate, settled=True):
         """K steps queued back to back between two HIP events on the launch stream: their distance
         / K is the average duration of a step's launches.  A step that has several phases (append,
         prefill, decode) also carries events between the phases, but only on ten of the steps: an
         event costs a few microseconds of stream time."""
+        if settled:
+            settle(lambda i: step(i if rotate else 0))
         for i in range(warmup):
             step(i if rotate else 0)
         torch.cuda.synchronize()
@@ -170,6 +188,7 @@ def run_decode_config(name, steps, warmup, dev):
 
     # the same loop over one pool (every step re-reads what the previous one read): kept beside
     # the rotating figure, which is the one the headline uses
+    wall_idle, _, region_idle, _ = timed_loop(rotate=True, settled=False)       # straight after set-up
     wall_1, _, region_1, evs_1 = timed_loop(rotate=False)
     wall, t_enqueue, region, evs = timed_loop(rotate=True)
     planned = None
@@ -187,6 +206,7 @@ def run_decode_config(name, steps, warmup, dev):
             kp, vp = pools[i % len(pools)]
             paged_attention_step(plan, out_all, w.query, w.new_key, w.new_value, kp, vp, w.scale, w.k_scale, w.v_scale)
 
+        settle(planned_step)
         for i in range(warmup):
             planned_step(i)
         torch.cuda.synchronize()
@@ -286,7 +306,9 @@ def run_decode_config(name, steps, warmup, dev):
     routed_small = (S - npre) * mb * w.shape.block_size <= ops.set_small_decode_tokens(-1)
     res = {
         "workload": name, "ms_per_step": (planned["wall"] if planned else wall) / steps * 1e3,
-        "pools_in_rotation": len(pools),
+        "pools_in_rotation": len(pools), "settle_ms": settle_ms,
+        "from_idle": {"ms_per_step": wall_idle / steps * 1e3, "device_us_per_step": region_idle * 1e6,
+                      "note": "the same K steps after only the W warm-up steps, the part coming out of idle"},
         "single_pool": {"ms_per_step": wall_1 / steps * 1e3, "decode_us": t_dec_1 * 1e6,
                         "decode_frac_hbm_peak": w.decode_kv_bytes() / t_dec_1 / 1e9 / HBM_PEAK_GBS,
                         "note": "the same loop re-reading one pool every step"},
@@ -976,7 +998,7 @@ def main():
                              "mixed_serial", "mixed_streams", "mixed_planned"],
                     help="profiling target: launch just this kernel --steps times (no JSON line)")
     ap.add_argument("--settle-ms", type=float, default=30.0,
-                    help="with --only: untimed launches for this long before the timed ones")
+                    help="untimed steps (launches, with --only) for this long before the warm-up and timed ones")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on one GPU only (asked for --gpus {args.gpus}); "
@@ -994,7 +1016,7 @@ def main():
     if args.only:
         profile_target(args.only, args.steps, args.warmup, dev, args.settle_ms)
         return
-    main_res, w = run_decode_config("llama3_8b_decode", args.steps, args.warmup, dev)
+    main_res, w = run_decode_config("llama3_8b_decode", args.steps, args.warmup, dev, args.settle_ms)
     s = w.shape
     line = {
         "metric": METRIC,
@@ -1002,6 +1024,9 @@ def main():
         "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": main_res["ms_per_step"],
+        # untimed steps of the same kind for this long before the W warm-up steps (an idle part's clock
+        # takes that long to come up); the K steps timed without them are in "from_idle"
+        "settle_ms": args.settle_ms, "from_idle": main_res["from_idle"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "llama3_8b_decode: batch 64, 32 query / 8 KV heads, head_dim 128, "
@@ -1041,8 +1066,8 @@ def main():
     if not args.no_extra:
         extra = []
         for name in ("decode_fp32_small", "long_context_skewed", "chunked_prefill_mixed",
-                     "llama3_70b_decode_fp8", "llama32_1b_decode"):
-            r, ww = run_decode_config(name, args.steps, args.warmup, dev)
+                     "llama32_1b_decode", "llama3_70b_decode_fp8"):
+            r, ww = run_decode_config(name, args.steps, args.warmup, dev, args.settle_ms)
             if not args.no_cpu:
                 # the reference's CPU path on the same batch, in the workload's own dtype (fp32 for
                 # the small anchor shape, which is defined on that path); a few seconds each
