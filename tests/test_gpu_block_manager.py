@@ -10,6 +10,7 @@ import numpy as np
 import pytest
 import torch
 
+from aicomp_amd import ops
 from aicomp_amd.block_manager import StepPlanner, paged_attention_step
 from oracle import paged_kv_oracle as orc
 from helpers import assert_close_attn, raw, to_f64
@@ -104,3 +105,86 @@ def test_serving_loop_with_preemption(device):
 def test_serving_loop_fp8(device):
     checked, pre, dec, p = run_serving(device, torch.float8_e4m3fn, steps=40, seed=2)
     assert pre >= 5 and dec >= 50
+
+
+@pytest.mark.parametrize("hq,hkv,d,dtype", [(8, 2, 128, torch.bfloat16), (16, 2, 64, torch.bfloat16), (4, 4, 128, torch.float16),
+                                            (6, 2, 64, torch.bfloat16), (16, 1, 128, torch.bfloat16)])
+def test_mixed_step_one_launch_equals_separate_kernels_random_mixes(device, monkeypatch, hq, hkv, d, dtype):
+    """paged_attention_step on random mixed steps (1 to 5 chunks of 1 to 200 tokens over priors of 0
+    to 600 tokens, 1 to 20 decode rows of 1 to 900 tokens), group sizes that pack into a column
+    group (4, 8, 16), that do not (3) and no grouping at all: the one-launch route against the
+    prefill and decode kernels.  Pools bit for bit, chunk rows bit for bit when the same kernel
+    variant ran them, decode rows and the rest within the attention tolerance; every row finite
+    over pools that start as NaN."""
+    from aicomp_amd.block_manager import StepPlan
+    rng = np.random.default_rng(hq * 100 + d)
+    g = torch.Generator().manual_seed(int(rng.integers(1 << 30)))
+    took_one = 0
+    for trial in range(6):
+        npre, ndec = int(rng.integers(1, 6)), int(rng.integers(1, 21))
+        news = [int(rng.integers(1, 201)) for _ in range(npre)]
+        news[0] = max(news[0], 130)                                   # a chunk long enough for two column groups
+        news = sorted(news, reverse=True) + [1] * ndec
+        ctx = [int(rng.integers(0, 601)) + n for n in news[:npre]] + [int(rng.integers(1, 901)) for _ in range(ndec)]
+        S, T = len(news), sum(news)
+        need = [-(-c // 16) for c in ctx]
+        nb = sum(need) + 2
+        perm = rng.permutation(nb - 1)
+        table = np.zeros((S, max(need)), dtype=np.int32)
+        at = 0
+        for s in range(S):
+            table[s, :need[s]] = perm[at:at + need[s]]
+            at += need[s]
+        cu = np.concatenate([[0], np.cumsum(news)]).astype(np.int32)
+        pos = np.concatenate([np.arange(c - n, c) for c, n in zip(ctx, news)])
+        seq_of = np.repeat(np.arange(S), news)
+        slots = table[seq_of, pos // 16].astype(np.int64) * 16 + pos % 16
+
+        def pools():
+            k = torch.full((nb, hkv, 16, d), float("nan"), dtype=dtype, device=device)
+            v = torch.full((nb, hkv, 16, d), float("nan"), dtype=dtype, device=device)
+            # the prior context of every sequence, the same in both runs
+            gg = torch.Generator().manual_seed(trial)
+            for s in range(S):
+                prior = ctx[s] - news[s]
+                if prior:
+                    p = np.arange(prior)
+                    sl = torch.from_numpy(table[s, p // 16].astype(np.int64) * 16 + p % 16).to(device)
+                    kk = (torch.randn(prior, hkv, d, generator=gg) * 0.5).to(dtype).to(device)
+                    vv = (torch.randn(prior, hkv, d, generator=gg) * 0.5).to(dtype).to(device)
+                    ops.kv_append(kk, vv, k, v, sl)
+            return k, v
+
+        plan = StepPlan(seq_ids=list(range(S)), num_prefill_seqs=npre, new_lens=np.asarray(news, dtype=np.int32),
+                        max_q_len=max(news[:npre]), total_new_tokens=T, block_table=torch.from_numpy(table).to(device),
+                        context_lens=torch.tensor(ctx, dtype=torch.int32, device=device),
+                        cu_q_lens=torch.from_numpy(cu).to(device), slot_mapping=torch.from_numpy(slots).to(device),
+                        positions=None, preempted=[], host_context_lens=np.asarray(ctx), host_cu_q_lens=cu)
+        q = torch.randn(T, hq, d, generator=g).to(dtype).to(device)
+        kn = (torch.randn(T, hkv, d, generator=g) * 0.5).to(dtype).to(device)
+        vn = (torch.randn(T, hkv, d, generator=g) * 0.5).to(dtype).to(device)
+        outs = []
+        for one in (True, False):
+            monkeypatch.setattr(StepPlan, "ONE_LAUNCH_MAX_ROWS", 128 if one else 0)
+            plan._prefill_items = None
+            k_pool, v_pool = pools()
+            out = torch.full((T, hq, d), float("nan"), dtype=dtype, device=device)
+            used = plan.step_items(q, k_pool) is not None
+            assert used == one
+            paged_attention_step(plan, out, q, kn, vn, k_pool, v_pool, 1 / math.sqrt(d))
+            torch.cuda.synchronize()
+            outs.append((out, k_pool, v_pool))
+        took_one += 1
+        (a, ka, va), (b, kb, vb) = outs
+        t_pre = int(cu[npre])
+        live = torch.zeros(nb * 16, dtype=torch.bool, device=device)
+        for s in range(S):
+            p = np.arange(ctx[s])
+            live[torch.from_numpy(table[s, p // 16].astype(np.int64) * 16 + p % 16).to(device)] = True
+        rows = lambda t: t.permute(0, 2, 1, 3).reshape(nb * 16, hkv, d)[live].view(torch.int16)
+        assert torch.equal(rows(ka), rows(kb)) and torch.equal(rows(va), rows(vb))
+        assert torch.isfinite(a.float()).all() and torch.isfinite(b.float()).all()
+        assert torch.equal(a[:t_pre].view(torch.int16), b[:t_pre].view(torch.int16)), f"trial {trial}: chunk rows"
+        err = (a[t_pre:].float() - b[t_pre:].float()).abs()
+        assert bool(((err <= 1e-2) | (err <= 2e-2 * b[t_pre:].float().abs())).all()), f"trial {trial}: {err.max().item():.3e}"
+    assert took_one == 6
