@@ -15,6 +15,7 @@
 
 #include <ATen/ATen.h>
 #include <ATen/hip/EmptyTensor.h>
+#include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/csrc/autograd/python_variable.h>
 
@@ -129,6 +130,7 @@ PyObject* decode_step(PyObject*, PyObject* const* args, Py_ssize_t nargs) {
             FAIL("key/value must both be [%d, %d or %d*group, 1, %d] of the query dtype on its device", L->B, L->hkv,
                  L->hkv, L->d);
         if (position < 0 || position + 1 >= L->ctx_count) FAIL("ctx_rows does not hold row %lld", (long long)(position + 1));
+        const c10::DeviceGuard guard(L->dev);              // launches go to the layer's device, whatever is current
         const at::Tensor query = q_in.is_contiguous() ? q_in : q_in.contiguous();
         at::Tensor k = key, v = value;
         if (k.stride(3) != 1 || k.strides() != v.strides()) { k = k.contiguous(); v = v.contiguous(); }

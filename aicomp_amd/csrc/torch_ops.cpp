@@ -18,6 +18,7 @@
 // (kv_cache.py:372-403) -> [B, Hq, 1, D].
 #include <ATen/ATen.h>
 #include <ATen/hip/HIPContext.h>
+#include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/library.h>
 
@@ -92,6 +93,7 @@ void kv_append(const at::Tensor& key, const at::Tensor& value, at::Tensor& k_poo
                const at::Tensor& slot_mapping, const c10::optional<at::Tensor>& k_scale,
                const c10::optional<at::Tensor>& v_scale) {
     const Pools p = check_pools(k_pool, v_pool);
+    const c10::DeviceGuard guard(k_pool.device());          // launches go to the tensors' device, whatever is current
     TORCH_CHECK(key.dim() == 3 && key.sizes() == value.sizes() && key.scalar_type() == value.scalar_type(),
                 "key/value must both be [T, Hkv, D]; got ", key.sizes(), " and ", value.sizes());
     TORCH_CHECK(key.size(1) == p.hkv && key.size(2) == p.d, "key is ", key.sizes(), " but the pool holds [", p.hkv,
@@ -145,6 +147,7 @@ void decode_impl(at::Tensor& out, const at::Tensor& query, const at::Tensor* new
                  const c10::optional<at::Tensor>& v_scale, int64_t partition_size,
                  const c10::optional<at::Tensor>& workspace) {
     const Pools p = check_pools(k_pool, v_pool);
+    const c10::DeviceGuard guard(k_pool.device());
     TORCH_CHECK(query.dim() == 3 && out.sizes() == query.sizes() && out.scalar_type() == query.scalar_type(),
                 "out/query must both be [B, Hq, D]; got ", out.sizes(), " and ", query.sizes());
     const int B = (int)query.size(0), hq = (int)query.size(1);
@@ -202,6 +205,7 @@ void paged_prefill_attn(at::Tensor& out, const at::Tensor& query, const at::Tens
                         double scale, int64_t max_q_len, const c10::optional<at::Tensor>& k_scale,
                         const c10::optional<at::Tensor>& v_scale, const c10::optional<at::Tensor>& items) {
     const Pools p = check_pools(k_pool, v_pool);
+    const c10::DeviceGuard guard(k_pool.device());
     TORCH_CHECK(query.dim() == 3 && out.sizes() == query.sizes() && out.scalar_type() == query.scalar_type(),
                 "out/query must both be [T, Hq, D]; got ", out.sizes(), " and ", query.sizes());
     TORCH_CHECK(query.size(2) == p.d, "query head_dim ", query.size(2), " != pool head_dim ", p.d);
@@ -235,6 +239,7 @@ at::Tensor decode_step(const at::Tensor& query_in, const at::Tensor& key, const 
                        at::Tensor& v_pool, const at::Tensor& block_table, const at::Tensor& ctx_rows, int64_t position,
                        int64_t group, double scale, const c10::optional<at::Tensor>& workspace) {
     const Pools p = check_pools(k_pool, v_pool);
+    const c10::DeviceGuard guard(k_pool.device());
     TORCH_CHECK(query_in.dim() == 4 && query_in.size(2) == 1 && query_in.size(3) == p.d &&
                 query_in.device() == k_pool.device(),
                 "query must be a [B, Hq, 1, ", p.d, "] tensor on ", k_pool.device(), "; got ", query_in.sizes());
