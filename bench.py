@@ -1065,8 +1065,8 @@ def main():
     torch.cuda.empty_cache()
     if not args.no_extra:
         extra = []
-        for name in ("decode_fp32_small", "long_context_skewed", "chunked_prefill_mixed",
-                     "llama32_1b_decode", "llama3_70b_decode_fp8"):
+        for name in ("decode_fp32_small", "llama32_1b_decode", "long_context_skewed", "chunked_prefill_mixed",
+                     "llama3_70b_decode_fp8"):
             r, ww = run_decode_config(name, args.steps, args.warmup, dev, args.settle_ms)
             if not args.no_cpu:
                 # the reference's CPU path on the same batch, in the workload's own dtype (fp32 for
