@@ -344,3 +344,16 @@ def test_prefill_with_a_caller_ranked_item_list_equals_grid_order(device, dtype,
                          c["ks"], c["vs"], torch.from_numpy(items).to(device))
     torch.cuda.synchronize()
     assert torch.equal(bits(out2), bits(plain))
+
+
+def test_item_list_longer_than_a_grid_dimension_is_ignored(device):
+    """More than 65535 pairs do not fit the launch grid's second dimension: the call then walks the
+    whole grid as the plain call does (the header says so), whatever the list holds."""
+    c = build_case(device, [5, 40], [70, 33], 8, 2, 128, seed=9)
+    plain = run(c, max_q_len=70)
+    items = torch.full((70000, 2), -7, dtype=torch.int32, device=device)
+    out = torch.full_like(c["q"], float("nan"))
+    ops.paged_prefill_attn(out, c["q"], c["k_pool"], c["v_pool"], c["table"], c["ctx"], c["cu"], c["scale"],
+                           max_q_len=70, items=items)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), plain.view(torch.int16))
