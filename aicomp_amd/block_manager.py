@@ -273,6 +273,9 @@ class _Staging:
         self.nbytes = nbytes
         self.host = [torch.empty(nbytes, dtype=torch.uint8, pin_memory=self.cuda) for _ in range(depth)]
         self.dev = [torch.empty(nbytes, dtype=torch.uint8, device=device) for _ in range(depth)] if self.cuda else self.host
+        # typed views of the device buffers, made once: a plan's tensors are then one slice each
+        self.dev32 = [d[:nbytes // 8 * 8].view(torch.int32) for d in self.dev]
+        self.dev64 = [d[:nbytes // 8 * 8].view(torch.int64) for d in self.dev]
         self.done = [torch.cuda.Event() if self.cuda else None for _ in range(depth)]
         self.used = [False] * depth
         self.i = 0
@@ -284,13 +287,12 @@ class _Staging:
             self.done[i].synchronize()          # the copy that last read this host buffer
         return i
 
-    def upload(self, i: int, nbytes: int) -> torch.Tensor:
-        if not self.cuda:
-            return self.host[i]
-        self.dev[i][:nbytes].copy_(self.host[i][:nbytes], non_blocking=True)
-        self.done[i].record()
-        self.used[i] = True
-        return self.dev[i]
+    def upload(self, i: int, nbytes: int) -> int:
+        if self.cuda:
+            self.dev[i][:nbytes].copy_(self.host[i][:nbytes], non_blocking=True)
+            self.done[i].record()
+            self.used[i] = True
+        return i
 
 
 class StepPlanner:
@@ -580,16 +582,17 @@ class StepPlanner:
                              host_context_lens=cl, host_cu_q_lens=cu, host_slot_mapping=slot, host_positions=posn)
             check_plan(probe, self.alloc.num_blocks, BS)       # raises before anything reaches the device
         self._len[rows] = cl
-        d = self._staging.upload(i, end)
-        dv = d[:end]
+        self._staging.upload(i, end)
+        d32, d64 = self._staging.dev32[i], self._staging.dev64[i]      # (every offset is a multiple of its element size)
+        ids = self._id_of
         return StepPlan(
-            seq_ids=[self._id_of[int(r)] for r in rows], num_prefill_seqs=npre, new_lens=new_lens,
+            seq_ids=[ids[r] for r in rows.tolist()], num_prefill_seqs=npre, new_lens=new_lens,
             max_q_len=int(new_lens[:npre].max()) if npre else 0, total_new_tokens=T,
-            block_table=dv[off_bt:off_cl].view(torch.int32).view(S, MB),
-            context_lens=dv[off_cl:off_cu].view(torch.int32),
-            cu_q_lens=dv[off_cu:end].view(torch.int32),
-            slot_mapping=dv[:off_pos].view(torch.int64),
-            positions=dv[off_pos:off_bt].view(torch.int64),
+            block_table=d32[off_bt // 4:off_cl // 4].view(S, MB),
+            context_lens=d32[off_cl // 4:off_cu // 4],
+            cu_q_lens=d32[off_cu // 4:end // 4],
+            slot_mapping=d64[:T],
+            positions=d64[T:2 * T],
             preempted=preempted,
             host_block_table=bt.copy(), host_context_lens=cl.copy(), host_cu_q_lens=cu.copy(),
             host_slot_mapping=slot.copy(), host_positions=posn.copy(),
