@@ -369,7 +369,7 @@ def prefill_items(context_lens, new_lens, tile_positions: int, num_head_groups: 
     n = order.size
     per_round = num_cus // num_head_groups if num_cus > 0 and num_head_groups > 0 and num_cus % num_head_groups == 0 else 0
     if per_round and per_round < n <= 2 * per_round:
-        # round 0 takes the per_round most expensive tiles in falling order, round 1 the rest in rising order
+        # the first pass over the CUs takes the per_round most expensive tiles in falling order, the second the rest in rising order
         order = np.concatenate([order[:per_round], order[per_round:][::-1]])
     return np.stack([seq[order], q[order]], axis=1).astype(np.int32)
 
